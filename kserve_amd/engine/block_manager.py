@@ -237,6 +237,20 @@ class BlockManager:
             table.append(blk)
         request.block_table = table
 
+    def extend_to(self, request: Request, num_tokens: int) -> None:
+        """Grow (or create) the request's table to hold ``num_tokens``."""
+        table = self._tables.get(request.request_id)
+        if table is None:
+            table = []
+            self._tables[request.request_id] = table
+            self._seq += 1
+            self._table_seq[request.request_id] = self._seq
+        while len(table) * self.block_size < num_tokens:
+            blk = self._take_block()
+            self._refcount[blk] = 1
+            table.append(blk)
+        request.block_table = table
+
     def _slots_free_in_last_block(self, request: Request) -> int:
         table = self._tables.get(request.request_id)
         if not table:

@@ -168,6 +168,177 @@ class ModelConfig:
 
 
 @dataclass
+class AttentionMixerSpec:
+    """Softmax attention sublayer with grouped KV heads. Independent query/key
+    and value head sizes; ``scale`` multiplies q.k; the query temperature
+    1 + coef * ln(floor((pos+1)/every) + 1) is off when ``q_temp_every`` is 0."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    q_temp_coef: float = 0.0
+    q_temp_every: int = 0
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "AttentionMixerSpec":
+        qt = d.get("q_temp") or {}
+        return cls(
+            heads=int(d["heads"]),
+            kv_heads=int(d.get("kv_heads", d["heads"])),
+            dim=int(d["dim"]),
+            vdim=int(d.get("vdim", d["dim"])),
+            scale=float(d["scale"]),
+            q_temp_coef=float(qt.get("coef", 0.0)),
+            q_temp_every=int(qt.get("every", 0)),
+        )
+
+
+@dataclass
+class SSMMixerSpec:
+    """State-space (Mamba-2) sublayer: ``heads`` heads of ``vdim`` channels,
+    state size ``state`` per channel, B/C shared per ``groups``, a causal
+    convolution of ``conv`` taps, and an output norm in ``norm_groups``
+    equal parts."""
+
+    heads: int
+    vdim: int
+    state: int
+    groups: int = 1
+    conv: int = 4
+    norm_groups: int = 1
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+    @property
+    def proj_width(self) -> int:
+        # [z | x | B | C | dt]
+        return 2 * self.inner + 2 * self.groups * self.state + self.heads
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "SSMMixerSpec":
+        return cls(
+            heads=int(d["heads"]),
+            vdim=int(d["vdim"]),
+            state=int(d["state"]),
+            groups=int(d.get("groups", 1)),
+            conv=int(d.get("conv", 4)),
+            norm_groups=int(d.get("norm_groups", 1)),
+        )
+
+
+@dataclass
+class GLUSpec:
+    """Dense gated feed-forward with clamped branches."""
+
+    ff: int
+    limit: float
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "GLUSpec":
+        kind = d.get("kind", "dense")
+        if kind != "dense":
+            raise ValueError(f"unsupported feed-forward kind {kind!r}")
+        return cls(ff=int(d["ff"]), limit=float(d["limit"]))
+
+
+@dataclass
+class HybridLayerSpec:
+    """One pre-norm layer: a mixer made of an attention branch and/or a
+    state-space branch reading the same normed input (outputs summed with
+    their scales), then an optional feed-forward."""
+
+    kind: str
+    attention: Optional[AttentionMixerSpec] = None
+    ssm: Optional[SSMMixerSpec] = None
+    attention_scale: float = 1.0
+    ssm_scale: float = 1.0
+    mlp: Optional[GLUSpec] = None
+
+
+@dataclass
+class HybridModelConfig:
+    """Decoder made of a per-layer list of mixers (Merulorn design): layers
+    may differ in kind and in every size, so nothing here is per-model."""
+
+    vocab_size: int
+    hidden_size: int
+    layers: list
+    rms_norm_eps: float = 1e-5
+    embedding_scale: float = 1.0
+    dtype: str = "bfloat16"
+    model_name: str = "merulorn"
+    architecture: str = "Merulorn"
+    # fields the engine reads on every model config
+    num_local_experts: int = 0
+    sliding_window: Optional[int] = None
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def has_recurrent_state(self) -> bool:
+        return any(l.ssm is not None for l in self.layers)
+
+    def kv_bytes_per_block(self, block_size: int, itemsize: int) -> int:
+        return sum(
+            l.attention.kv_heads * (l.attention.dim + l.attention.vdim)
+            for l in self.layers
+            if l.attention is not None
+        ) * block_size * itemsize
+
+    @classmethod
+    def from_dict(cls, cfg: dict, model_name: str = "merulorn") -> "HybridModelConfig":
+        layers = []
+        for entry in cfg["layers"]:
+            kind = entry["type"]
+            mixer = entry["mixer"]
+            mlp = GLUSpec.from_dict(entry["mlp"]) if entry.get("mlp") else None
+            if kind == "mamba2":
+                layers.append(
+                    HybridLayerSpec(kind, ssm=SSMMixerSpec.from_dict(mixer), mlp=mlp)
+                )
+            elif kind == "parallel":
+                layers.append(
+                    HybridLayerSpec(
+                        kind,
+                        attention=AttentionMixerSpec.from_dict(mixer["left"]),
+                        ssm=SSMMixerSpec.from_dict(mixer["right"]),
+                        attention_scale=float(mixer.get("left_scale", 1.0)),
+                        ssm_scale=float(mixer.get("right_scale", 1.0)),
+                        mlp=mlp,
+                    )
+                )
+            else:
+                raise ValueError(f"unknown layer type {kind!r}")
+        return cls(
+            vocab_size=int(cfg["vocab"]),
+            hidden_size=int(cfg["width"]),
+            layers=layers,
+            rms_norm_eps=float(cfg.get("norm", {}).get("eps", 1e-5)),
+            embedding_scale=float(cfg.get("embedding", {}).get("scale", 1.0)),
+            model_name=model_name,
+            architecture=cfg.get("architecture", "Merulorn"),
+        )
+
+    @classmethod
+    def from_hf_config(cls, config_path: str) -> "HybridModelConfig":
+        with open(config_path) as f:
+            cfg = json.load(f)
+        return cls.from_dict(
+            cfg, model_name=os.path.basename(os.path.dirname(config_path)) or "merulorn"
+        )
+
+
+@dataclass
 class CacheConfig:
     """Paged-KV cache sizing. Defaults size the pool from the 288 GB HBM3E
     budget after weights (MI355X-first: large pools, big batches)."""

@@ -189,6 +189,7 @@ class LLMEngine:
         self.scheduler = Scheduler(
             config.scheduler, config.cache, num_blocks,
             num_cpu_blocks=self.runner.num_cpu_blocks,
+            num_state_slots=self.runner.num_state_slots,
         )
         self.sampler = Sampler(self.device, config.seed)
         self.lora_manager = None
@@ -226,9 +227,11 @@ class LLMEngine:
         )
 
     def _build_model(self) -> LlamaForCausalLM:
+        from kserve_amd.models.registry import build_model
+
         cfg = self.config
         with torch.device(self.device):
-            model = LlamaForCausalLM(cfg.model, device=str(self.device))
+            model = build_model(cfg.model, device=str(self.device))
         if cfg.model_path:
             from kserve_amd.engine.weights import load_safetensors_weights
 
@@ -531,6 +534,37 @@ class LLMEngine:
                 self.draft.release(req.request_id)
         LLM_KV_USAGE.set(self.scheduler.block_manager.usage)
         return outputs
+
+    # -- replaying a fixed schedule ---------------------------------------------
+    @torch.no_grad()
+    def forced_step(self, items, logit_rows) -> Optional[torch.Tensor]:
+        """Run exactly ``items`` = [(request, num_tokens)] as one batch (see
+        Scheduler.schedule_forced) without sampling, and return the logits of
+        the flat token rows ``logit_rows`` (None when empty). Decode-only
+        batches take the decode path (captured graphs when enabled), anything
+        else the paged-context prefill path — the same two paths ``step()``
+        drives."""
+        batch = self.scheduler.schedule_forced(items)
+        bm = self.scheduler.block_manager
+        if batch.is_prefill:
+            # the forward must run even when no logits are asked for: it
+            # writes the KV pages and advances the recurrent state
+            logits = self.runner.execute_prefill(
+                batch, bm, logit_rows=list(logit_rows)
+            )
+        else:
+            logits = self.runner.execute_decode(batch, bm)
+            if logits is not None:
+                logits = logits[list(logit_rows)]
+        for req, n in zip(batch.requests, batch.num_scheduled_tokens):
+            req.num_computed_tokens += n
+        return logits if len(logit_rows) else None
+
+    def release(self, requests) -> None:
+        """Return the pages and state slots of requests that are done."""
+        self.scheduler.finish_requests(requests)
+        for req in requests:
+            self.runner.release_request(req.request_id)
 
     def _sample_tokens(self, logits, sample_reqs) -> List[int]:
         """Sample on the last pipeline stage and broadcast the token ids so

@@ -66,6 +66,13 @@ class ModelRunner:
         )
         # multi-LoRA (set by LLMEngine.register_lora)
         self.lora_manager = None
+        # models that describe their own per-layer cache (mixed attention /
+        # recurrent layers) instead of the uniform llama KV layout
+        self._layout = (
+            model.cache_layout() if hasattr(model, "cache_layout") else None
+        )
+        self.num_state_slots = 0
+        self._arange: Optional[torch.Tensor] = None
 
     # -- KV cache -----------------------------------------------------------
     def profile_and_allocate_kv(self) -> int:
@@ -80,14 +87,19 @@ class ModelRunner:
                 free_bytes * self.config.cache.gpu_memory_utilization
             ) - (2 << 30)
             kv_itemsize = self.config.cache.cache_torch_dtype(dtype).itemsize
-            # kv_bytes_per_token_per_layer assumes bf16 (2 B); rescale
-            per_block_bytes = (
-                m.kv_bytes_per_token_per_layer
-                * kv_itemsize
-                * self.config.cache.block_size
-                * self._num_local_layers()
-                // (tp * 2)
-            )
+            if hasattr(m, "kv_bytes_per_block"):
+                per_block_bytes = max(
+                    1, m.kv_bytes_per_block(self.config.cache.block_size, kv_itemsize)
+                )
+            else:
+                # kv_bytes_per_token_per_layer assumes bf16 (2 B); rescale
+                per_block_bytes = (
+                    m.kv_bytes_per_token_per_layer
+                    * kv_itemsize
+                    * self.config.cache.block_size
+                    * self._num_local_layers()
+                    // (tp * 2)
+                )
             num_blocks = self.config.cache.num_gpu_blocks or max(
                 budget // per_block_bytes,
                 16,
@@ -100,7 +112,63 @@ class ModelRunner:
     def _num_local_layers(self) -> int:
         return getattr(self.model, "num_local_layers", self.config.model.num_layers)
 
+    def _arange_i32(self, n: int) -> torch.Tensor:
+        if self._arange is None or self._arange.shape[0] < n:
+            self._arange = torch.arange(
+                max(n, 4096), dtype=torch.int32, device=self.device
+            )
+        return self._arange[:n]
+
+    def _allocate_layout(self, num_blocks: int):
+        """Per-layer caches for models with ``cache_layout()``: KV pages only
+        for layers with attention, recurrent-state pools (one row per state
+        slot) for layers that carry state. Pools are uninitialised: pages are
+        bounded by context lengths, and a sequence starting at position 0
+        never reads its slot."""
+        from kserve_amd.models.mixers import LayerCache
+
+        if self.config.cache.kv_cache_dtype != "auto":
+            raise ValueError("this model keeps its KV pages in the model dtype")
+        if self.config.cache.num_cpu_blocks or self.config.cache.cpu_offload_bytes:
+            raise ValueError("recurrent state has no host offload tier")
+        if self.config.cache.enable_prefix_caching:
+            raise ValueError(
+                "prefix caching needs the recurrent state at the cached "
+                "boundary, which is not kept"
+            )
+        bs = self.config.cache.block_size
+        dtype = self.model.dtype
+        # slot 0 is scratch for padded graph lanes
+        slots = self.config.scheduler.max_num_seqs + 1
+        alloc = torch.empty if self.is_cuda else torch.zeros
+        caches = []
+        kv_bytes = state_bytes = 0
+        for kv, state in self._layout:
+            k = v = conv = ssm = None
+            if kv is not None:
+                g, d, dv = kv
+                k = alloc((num_blocks, g, bs, d), dtype=dtype, device=self.device)
+                v = alloc((num_blocks, g, bs, dv), dtype=dtype, device=self.device)
+                kv_bytes += k.numel() * k.itemsize + v.numel() * v.itemsize
+            if state:
+                shape, dt = state["conv"]
+                conv = alloc((slots, *shape), dtype=dt, device=self.device)
+                shape, dt = state["ssm"]
+                ssm = alloc((slots, *shape), dtype=dt, device=self.device)
+                state_bytes += conv.numel() * conv.itemsize + ssm.numel() * ssm.itemsize
+            caches.append(LayerCache(k, v, conv, ssm))
+        self.kv_caches = caches
+        self.num_gpu_blocks = num_blocks
+        self.num_state_slots = slots if state_bytes else 0
+        logger.info(
+            "Layer caches: %d KV blocks x %d tokens (%.2f GiB), %d state slots (%.2f GiB)",
+            num_blocks, bs, kv_bytes / (1 << 30), slots, state_bytes / (1 << 30),
+        )
+
     def allocate_kv_cache(self, num_blocks: int):
+        if self._layout is not None:
+            self._allocate_layout(num_blocks)
+            return
         m = self.config.model
         kv_heads_local = max(1, m.num_kv_heads // max(1, self._tp_size()))
         shape = (
@@ -240,10 +308,21 @@ class ModelRunner:
             cu_seqlens=torch.tensor(cu, dtype=torch.int32, device=dev),
             max_seqlen=max_seqlen,
         )
+        if self._layout is not None:
+            counts = np.asarray(batch.num_scheduled_tokens, dtype=np.int64)
+            meta.seq_of_token = torch.from_numpy(
+                np.repeat(np.arange(len(counts), dtype=np.int32), counts)
+            ).to(dev, non_blocking=True)
+            meta.state_slots = torch.tensor(
+                [r.state_slot for r in batch.requests],
+                dtype=torch.int32, device=dev,
+            )
         # chunked-prefill resume: any request with context already in pages
         # must attend to it — switch to the paged-context attention path
-        if any(r.num_computed_tokens > 0 for r in batch.requests) and (
-            self.kv_caches and self.kv_caches[0][0].numel() > 0
+        # (models without an un-paged prefill kernel always take it)
+        if getattr(self.model, "paged_prefill_only", False) or (
+            any(r.num_computed_tokens > 0 for r in batch.requests)
+            and self.kv_caches and self.kv_caches[0][0].numel() > 0
         ):
             nb_per = [
                 -(-(r.num_computed_tokens + n) // bs)
@@ -282,6 +361,7 @@ class ModelRunner:
                 "positions": torch.empty(cap, dtype=torch.int64, pin_memory=pin),
                 "slot_mapping": torch.empty(cap, dtype=torch.int32, pin_memory=pin),
                 "context_lens": torch.empty(cap, dtype=torch.int32, pin_memory=pin),
+                "state_slots": torch.zeros(cap, dtype=torch.int32, pin_memory=pin),
                 "block_tables": torch.zeros(
                     (cap, mb), dtype=torch.int32, pin_memory=pin
                 ),
@@ -309,8 +389,10 @@ class ModelRunner:
         sm = pnp["slot_mapping"]
         ctx = pnp["context_lens"]
         btab = pnp["block_tables"]
+        ss = pnp["state_slots"]
         for i, req in enumerate(batch.requests):
             pos = req.num_computed_tokens
+            ss[i] = req.state_slot
             ii[i] = req.all_token_ids[pos]
             pp[i] = pos
             t = tables[i]
@@ -343,9 +425,20 @@ class ModelRunner:
             .contiguous(),
             context_lens=pin["context_lens"][:n].to(dev, non_blocking=True),
         )
+        if self._layout is not None:
+            self._decode_layout_meta(
+                meta, n, pin["state_slots"][:n].to(dev, non_blocking=True)
+            )
         input_ids = pin["input_ids"][:n].to(dev, non_blocking=True)
         pos = pin["positions"][:n].to(dev, non_blocking=True)
         return input_ids, pos, meta
+
+    def _decode_layout_meta(self, meta, n: int, state_slots) -> None:
+        """Decode is the flat-batch layout with one token per sequence."""
+        meta.cu_seqlens = self._arange_i32(n + 1)
+        meta.seq_of_token = self._arange_i32(n)
+        meta.max_seqlen = 1
+        meta.state_slots = state_slots
 
     def _lora_meta(self, batch: ScheduledBatch, per_request_rows: bool):
         """Contiguous (adapter_id, start_row, end_row) segments for the batch.
@@ -373,8 +466,12 @@ class ModelRunner:
 
     # -- execution ----------------------------------------------------------
     @torch.no_grad()
-    def execute_prefill(self, batch, block_manager) -> torch.Tensor:
+    def execute_prefill(self, batch, block_manager, logit_rows=None) -> torch.Tensor:
+        """Logits of each request's last scheduled token, or of the flat
+        token rows in ``logit_rows`` when given."""
         input_ids, positions, meta, sel = self.prepare_prefill(batch, block_manager)
+        if logit_rows is not None:
+            sel = torch.tensor(logit_rows, dtype=torch.int64, device=self.device)
         if self.lora_manager is not None and any(
             r.lora_id for r in batch.requests
         ):
@@ -474,6 +571,7 @@ class ModelRunner:
                 (max_bs, mb), dtype=torch.int32, device=dev
             ),
             "context_lens": torch.ones(max_bs, dtype=torch.int32, device=dev),
+            "state_slots": torch.zeros(max_bs, dtype=torch.int32, device=dev),
             # per-request sampling params (sampled-window variants)
             "temps": torch.ones(max_bs, dtype=torch.float32, device=dev),
             "top_p": torch.ones(max_bs, dtype=torch.float32, device=dev),
@@ -505,6 +603,8 @@ class ModelRunner:
                     block_tables=bt,
                     context_lens=buf["context_lens"][:bs],
                 )
+                if self._layout is not None:
+                    self._decode_layout_meta(meta, bs, buf["state_slots"][:bs])
                 hidden = self.model(
                     buf["input_ids"][:bs], pos, self.kv_caches, meta
                 )
@@ -559,6 +659,8 @@ class ModelRunner:
                 block_tables=bt,
                 context_lens=buf["context_lens"][:bs],
             )
+            if self._layout is not None:
+                self._decode_layout_meta(meta, bs, buf["state_slots"][:bs])
             hidden = self.model(
                 buf["input_ids"][:bs], pos, self.kv_caches, meta
             )
@@ -602,8 +704,12 @@ class ModelRunner:
             pnp["input_ids"][n:bucket] = 0
             pnp["positions"][n:bucket] = 0
             pnp["context_lens"][n:bucket] = 1
+            pnp["state_slots"][n:bucket] = 0
             pnp["block_tables"][n:bucket, :nb] = 0
         buf = self._graph_buffers
+        buf["state_slots"][:bucket].copy_(
+            pin["state_slots"][:bucket], non_blocking=True
+        )
         # single async H2D per tensor, pinned -> static graph buffers
         # (slot mapping is derived in-graph from block_tables + positions)
         buf["input_ids"][:bucket].copy_(pin["input_ids"][:bucket], non_blocking=True)
@@ -625,8 +731,12 @@ class ModelRunner:
             pnp["input_ids"][n:bucket] = 0
             pnp["positions"][n:bucket] = 0
             pnp["context_lens"][n:bucket] = 1
+            pnp["state_slots"][n:bucket] = 0
             pnp["block_tables"][n:bucket, :nb] = 0
         buf = self._graph_buffers
+        buf["state_slots"][:bucket].copy_(
+            pin["state_slots"][:bucket], non_blocking=True
+        )
         buf["input_ids"][:bucket].copy_(pin["input_ids"][:bucket], non_blocking=True)
         buf["positions"][:bucket].copy_(pin["positions"][:bucket], non_blocking=True)
         buf["context_lens"][:bucket].copy_(
@@ -770,6 +880,8 @@ class ModelRunner:
                 block_tables=bt,
                 context_lens=ctx,
             )
+            if self._layout is not None:
+                self._decode_layout_meta(meta_k, n, meta.state_slots)
             hidden = self.model(input_ids, positions, self.kv_caches, meta_k)
             logits = self.model.compute_logits(hidden)
             if sampled:

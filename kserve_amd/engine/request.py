@@ -61,6 +61,8 @@ class Request:
         self.block_table: List[int] = []
         # number of prompt tokens whose KV is already computed (chunked prefill)
         self.num_computed_tokens = 0
+        # row of the recurrent-state pools (0 = none / scratch)
+        self.state_slot = 0
         # multi-LoRA adapter id (0 = base model)
         self.lora_id = 0
         # guided decoding (engine/guided.py): per-request JSON machine

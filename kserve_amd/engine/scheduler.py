@@ -20,6 +20,7 @@ from typing import Deque, List, Optional
 from kserve_amd.engine.block_manager import BlockManager
 from kserve_amd.engine.config import CacheConfig, SchedulerConfig
 from kserve_amd.engine.request import Request, RequestStatus
+from kserve_amd.engine.state_manager import StateSlotManager
 from kserve_amd.metrics import LLM_NUM_RUNNING, LLM_NUM_WAITING, LLM_PREEMPTIONS
 
 
@@ -51,8 +52,14 @@ class Scheduler:
         cache_config: CacheConfig,
         num_gpu_blocks: int,
         num_cpu_blocks: int = 0,
+        num_state_slots: int = 0,
     ):
         self.config = scheduler_config
+        # recurrent-state models: one state slot per live request, taken at
+        # admission and returned with the KV blocks (0 = model has no state)
+        self.state_slots = (
+            StateSlotManager(num_state_slots) if num_state_slots else None
+        )
         self.block_manager = BlockManager(
             num_gpu_blocks, cache_config.block_size,
             num_cpu_blocks=num_cpu_blocks or cache_config.num_cpu_blocks,
@@ -98,8 +105,24 @@ class Scheduler:
                     q.remove(r)
                     self.block_manager.free(r)
                     self.block_manager.free_cpu(r)
+                    self._release_state(r)
                     return r
         return None
+
+    def _release_state(self, req: Request) -> None:
+        if self.state_slots is not None:
+            self.state_slots.free(req.request_id)
+            req.state_slot = 0
+
+    def _take_state(self, req: Request) -> bool:
+        """Give the request a state slot if the model needs one. False when
+        none is free (the request stays queued)."""
+        if self.state_slots is None or self.state_slots.has(req.request_id):
+            return True
+        if self.state_slots.num_free == 0:
+            return False
+        req.state_slot = self.state_slots.allocate(req.request_id)
+        return True
 
     @property
     def num_waiting(self) -> int:
@@ -137,6 +160,12 @@ class Scheduler:
             n_new = req.num_tokens - base_computed
             if len(self.running) + len(batch.requests) + 1 > self.config.max_num_seqs:
                 break
+            if (
+                self.state_slots is not None
+                and not self.state_slots.has(req.request_id)
+                and self.state_slots.num_free == 0
+            ):
+                break
             if n_new > token_budget:
                 if self.config.enable_chunked_prefill and token_budget > 0 and batch.total_tokens == 0:
                     n_new = token_budget
@@ -169,6 +198,7 @@ class Scheduler:
                     )
                     n_new = min(req.num_tokens - cached, capacity - cached)
             self.waiting.pop(0)
+            self._take_state(req)
             req.status = RequestStatus.RUNNING
             batch.requests.append(req)
             batch.num_scheduled_tokens.append(n_new)
@@ -211,7 +241,8 @@ class Scheduler:
             if total_needed <= self.block_manager.num_free_blocks:
                 break
             victim = scheduled.pop()  # newest in running order
-            if self.block_manager.can_swap_out(victim):
+            # recurrent state has no host tier: such models always recompute
+            if self.state_slots is None and self.block_manager.can_swap_out(victim):
                 batch.swap_out.extend(self._preempt_swap(victim))
             else:
                 self._preempt(victim)
@@ -232,6 +263,9 @@ class Scheduler:
         """
         LLM_PREEMPTIONS.inc()
         self.block_manager.free(req)
+        # the recurrent state goes with the pages: the re-prefill starts at
+        # position 0, which the kernels take as a zero state
+        self._release_state(req)
         req.num_computed_tokens = 0
         req.status = RequestStatus.PREEMPTED
         self._enqueue(req)
@@ -260,6 +294,48 @@ class Scheduler:
                 self.running.remove(req)
             self.block_manager.free(req)
             self.block_manager.free_cpu(req)
+            self._release_state(req)
+
+    # -- forced schedules ------------------------------------------------------
+    def schedule_forced(self, items) -> ScheduledBatch:
+        """One batch made of exactly the given (request, num_tokens) pairs:
+        the next ``num_tokens`` uncomputed tokens of each request, prompt
+        portions and single decode tokens side by side. Used to replay a
+        recorded schedule through the engine; admission control is the
+        caller's, so pages are taken down to the last free one. The batch is
+        a decode batch when every request brings one token onto an existing
+        context, else it runs through the paged-context prefill path."""
+        bm = self.block_manager
+        need = 0
+        for req, n in items:
+            if req.num_computed_tokens + n > req.num_tokens:
+                raise ValueError("scheduled more tokens than the request holds")
+            need += max(
+                0,
+                bm.blocks_needed(req.num_computed_tokens + n)
+                - len(bm.get_block_table(req)),
+            )
+            if self.state_slots is not None and not self.state_slots.has(
+                req.request_id
+            ) and self.state_slots.num_free == 0:
+                raise RuntimeError("Out of state slots")
+        if need > bm.num_free_blocks:
+            raise RuntimeError("Out of KV blocks")
+        all_decode = all(
+            n == 1 and req.num_computed_tokens > 0 for req, n in items
+        )
+        batch = ScheduledBatch(is_prefill=not all_decode)
+        for req, n in items:
+            if req in self.waiting:
+                self.waiting.remove(req)
+            if req not in self.running:
+                self.running.append(req)
+            req.status = RequestStatus.RUNNING
+            self._take_state(req)
+            bm.extend_to(req, req.num_computed_tokens + n)
+            batch.requests.append(req)
+            batch.num_scheduled_tokens.append(n)
+        return batch
 
     # -- multi-step decode windows -------------------------------------------
     # window length while admission is blocked: a waiting request was

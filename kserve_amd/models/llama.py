@@ -46,6 +46,11 @@ class AttentionMetadata:
     context_lens: Optional[torch.Tensor] = None  # [num_seqs] int32
     # multi-LoRA: per-batch adapter segments (engine/lora.LoRABatchMeta)
     lora: Optional[object] = None
+    # recurrent-state models: sequence index of every flat token, and the
+    # state-pool row of every sequence (decode: cu_seqlens = 0..n, one token
+    # per sequence)
+    seq_of_token: Optional[torch.Tensor] = None  # [num_tokens] int32
+    state_slots: Optional[torch.Tensor] = None  # [num_seqs] int32
 
 
 class LlamaAttention(nn.Module):

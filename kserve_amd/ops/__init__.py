@@ -23,8 +23,33 @@ except ImportError as e:  # pragma: no cover - exercised on GPU box
     _IMPORT_ERROR = str(e)
 
 
+# kernels of the 32-bit-residual / recurrent-state mechanisms (own module so
+# a model built from them compiles nothing else); carries the samplers too
+_SEQ = None
+_SEQ_IMPORT_ERROR: Optional[str] = None
+try:
+    import kserve_amd_seq_C as _SEQ
+except ImportError as e:  # pragma: no cover - exercised on GPU box
+    _SEQ_IMPORT_ERROR = str(e)
+
+
 def has_native() -> bool:
     return _C is not None
+
+
+def has_native_seq() -> bool:
+    return _SEQ is not None
+
+
+def _native_seq(op: str):
+    if _SEQ is None:
+        raise NoNativeExtension(op, f"(import error: {_SEQ_IMPORT_ERROR})")
+    return _SEQ
+
+
+def _native_sampling(op: str):
+    """The samplers are linked into every extension module."""
+    return _C if _C is not None else _native_seq(op)
 
 
 def _native(op: str):
@@ -165,10 +190,13 @@ def context_attention_varlen(
 
 def greedy_sample(logits: torch.Tensor) -> torch.Tensor:
     if logits.is_cuda:
+        if logits.dtype != torch.bfloat16:
+            # fp32 engines: the argmax must see every bit of the logits
+            return torch.argmax(logits, dim=-1)
         out = torch.empty(
             logits.shape[0], dtype=torch.int64, device=logits.device
         )
-        _native("greedy_sample").greedy_sample(out, logits)
+        _native_sampling("greedy_sample").greedy_sample(out, logits)
         return out
     return torch_ref.greedy_sample(logits)
 
@@ -191,16 +219,18 @@ def random_sample(
     """
     has_min_p = min_p is not None and bool((min_p > 0).any())
     if logits.is_cuda and seeds is not None and not has_min_p:
+        if logits.dtype != torch.bfloat16:
+            logits = logits.to(torch.bfloat16)  # the fused samplers' format
         out = torch.empty(
             logits.shape[0], dtype=torch.int64, device=logits.device
         )
         needs_trunc = bool((top_p < 1.0).any()) or bool((top_k > 0).any())
         if needs_trunc:
-            _native("random_sample").topk_topp_sample(
+            _native_sampling("random_sample").topk_topp_sample(
                 out, logits, temperatures, top_p, top_k.to(torch.int32), seeds
             )
         else:
-            _native("random_sample").gumbel_sample(
+            _native_sampling("random_sample").gumbel_sample(
                 out, logits, temperatures, top_k.to(torch.int32), seeds
             )
         return out
@@ -287,9 +317,140 @@ def topk_topp_sample_into(
     """Destination-passing form of the fused sampler for hipGraph capture
     (static out buffer, per-row device seeds; see model_runner
     _ensure_sampled_graph). GPU-only."""
-    _native("random_sample").topk_topp_sample(
+    _native_sampling("random_sample").topk_topp_sample(
         out, logits, temperatures, top_p,
         top_k if top_k.dtype == torch.int32 else top_k.to(torch.int32),
         seeds,
     )
     return out
+
+
+# -- 32-bit residual stream, recurrent state, fp32 attention -----------------
+
+def _f32_like(rows: int, cols: int, ref: torch.Tensor) -> torch.Tensor:
+    return torch.empty((rows, cols), dtype=torch.float32, device=ref.device)
+
+
+def embed_scale_sinpos(table, tokens, positions, inv_freq, scale: float):
+    """fp32 [T, width]: table[token] * scale + interleaved sin/cos of
+    position * inv_freq (the start of an fp32 residual stream)."""
+    if table.is_cuda:
+        out = _f32_like(tokens.shape[0], table.shape[1], table)
+        _native_seq("embed_scale_sinpos").embed_scale_sinpos(
+            out, table, tokens, positions, inv_freq, float(scale)
+        )
+        return out
+    return torch_ref.embed_scale_sinpos(table, tokens, positions, inv_freq, scale)
+
+
+def add_rms_norm_f32res(
+    residual, weight, eps: float, w_offset: float, out_dtype,
+    d0=None, s0: float = 1.0, d1=None, s1: float = 1.0,
+):
+    """residual (fp32, in place) += s0*d0 + s1*d1, then RMS norm with weight
+    (w_offset + w); returns the normed rows in ``out_dtype``."""
+    if residual.is_cuda:
+        out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+        _native_seq("add_rms_norm_f32res").add_rms_norm_f32res(
+            residual, d0, float(s0), d1, float(s1), weight, float(w_offset),
+            float(eps), out,
+        )
+        return out
+    return torch_ref.add_rms_norm_f32res(
+        residual, weight, eps, w_offset, out_dtype, d0, s0, d1, s1
+    )
+
+
+def gated_group_rms_norm(y, z, weight, eps: float, groups: int, out_dtype):
+    if y.is_cuda:
+        out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+        _native_seq("gated_group_rms_norm").gated_group_rms_norm(
+            out, y, z, weight, float(eps), int(groups)
+        )
+        return out
+    return torch_ref.gated_group_rms_norm(y, z, weight, eps, groups, out_dtype)
+
+
+def causal_conv_silu(
+    x_in, w, bias, conv_state, positions, seq_of_token, cu_seqlens, slots
+):
+    """Depthwise causal conv + silu over a flat varlen batch; reads and then
+    advances each sequence's conv history in ``conv_state[slot]``."""
+    if x_in.is_cuda:
+        out = _f32_like(x_in.shape[0], x_in.shape[1], x_in)
+        _native_seq("causal_conv_silu").causal_conv_silu(
+            out, x_in, w, bias, conv_state, positions, seq_of_token,
+            cu_seqlens, slots,
+        )
+        return out
+    return torch_ref.causal_conv_silu(
+        x_in, w, bias, conv_state, positions, cu_seqlens, slots
+    )
+
+
+def ssd_scan(
+    xbc, dt_raw, dt_bias, a_log, d_skip, state, positions, cu_seqlens, slots,
+    groups: int,
+):
+    """State-space scan; carries ``state[slot]`` ([heads, P, N] fp32)."""
+    if xbc.is_cuda:
+        heads, P = state.shape[1], state.shape[2]
+        y = _f32_like(xbc.shape[0], heads * P, xbc)
+        _native_seq("ssd_scan").ssd_scan(
+            y, xbc, dt_raw, dt_bias, a_log, d_skip, state, positions,
+            cu_seqlens, slots, int(groups),
+        )
+        return y
+    return torch_ref.ssd_scan(
+        xbc, dt_raw, dt_bias, a_log, d_skip, state, positions, cu_seqlens,
+        slots, groups,
+    )
+
+
+def qk_norm_temp_cache(
+    q, k, v, qw, kw, positions, slot_mapping, k_cache, v_cache, eps: float,
+    temp_coef: float, temp_every: int, heads: int,
+):
+    if q.is_cuda:
+        q_out = _f32_like(q.shape[0], q.shape[1], q)
+        _native_seq("qk_norm_temp_cache").qk_norm_temp_cache(
+            q_out, q, k, v, qw, kw, positions, slot_mapping, k_cache, v_cache,
+            float(eps), float(temp_coef), int(temp_every), int(heads),
+        )
+        return q_out
+    return torch_ref.qk_norm_temp_cache(
+        q, k, v, qw, kw, positions, slot_mapping, k_cache, v_cache, eps,
+        temp_coef, temp_every, heads,
+    )
+
+
+def ctx_attention_f32(
+    q, k_cache, v_cache, block_tables, cu_q, ctx_lens, scale: float,
+    max_q_len: int, heads: int, gate=None, out_dtype=torch.float32,
+):
+    if q.is_cuda:
+        out = torch.empty(
+            (q.shape[0], heads * v_cache.shape[3]), dtype=out_dtype,
+            device=q.device,
+        )
+        _native_seq("ctx_attention_f32").ctx_attention_f32(
+            out, q, k_cache, v_cache, block_tables, cu_q, ctx_lens, gate,
+            float(scale), int(max_q_len), int(heads),
+        )
+        return out
+    return torch_ref.ctx_attention_f32(
+        q, k_cache, v_cache, block_tables, cu_q, ctx_lens, scale, heads,
+        gate, out_dtype,
+    )
+
+
+def clamped_swiglu(x, alpha: float, limit: float):
+    if x.is_cuda:
+        out = torch.empty(
+            (*x.shape[:-1], x.shape[-1] // 2), dtype=x.dtype, device=x.device
+        )
+        _native_seq("clamped_swiglu").clamped_swiglu(
+            out, x, float(alpha), float(limit)
+        )
+        return out
+    return torch_ref.clamped_swiglu(x, alpha, limit)

@@ -1,8 +1,29 @@
 // SwiGLU activation: out = silu(gate) * up, input layout [rows, 2*d] = [gate|up].
 // Memory-bound elementwise; vectorized short8 (CDNA guide Appendix B).
-#include "common.h"
+//
+// clamped_swiglu: out = g * sigmoid(alpha * g) * (u + 1) with g = min(gate,
+// limit) and u = clamp(up, -limit, limit); same [gate|up] layout, either
+// activation dtype, fp32 arithmetic.
+#include "dtype_io.h"
 
 namespace {
+
+template <typename T>
+__global__ void clamped_swiglu_kernel(T* __restrict__ out,
+                                      const T* __restrict__ input,
+                                      const long rows, const int d,
+                                      const float alpha, const float limit) {
+  const long total = rows * d;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long row = idx / d;
+    const long col = idx % d;
+    const float g = fminf(ld_f32(input, row * 2 * d + col), limit);
+    const float u =
+        fminf(fmaxf(ld_f32(input, row * 2 * d + d + col), -limit), limit);
+    st_f32(out, idx, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+  }
+}
 
 __global__ void silu_and_mul_kernel(short* __restrict__ out,
                                     const short* __restrict__ input,
@@ -40,6 +61,25 @@ extern "C" hipError_t ks_silu_and_mul(void* out, const void* input, int rows,
   if (grid > 2048) grid = 2048;  // grid-stride (G11)
   hipLaunchKernelGGL(silu_and_mul_kernel, dim3(grid), dim3(256), 0, stream,
                      (short*)out, (const short*)input, rows, d);
+  HIP_CHECK_KERNEL();
+  return hipSuccess;
+}
+
+extern "C" hipError_t ks_clamped_swiglu(void* out, const void* input, int rows,
+                                        int d, float alpha, float limit,
+                                        int is_f32, hipStream_t stream) {
+  long total = (long)rows * d;
+  if (total == 0) return hipSuccess;
+  int grid = (int)((total + 255) / 256);
+  if (grid > 4096) grid = 4096;
+  if (is_f32)
+    hipLaunchKernelGGL(clamped_swiglu_kernel<float>, dim3(grid), dim3(256), 0,
+                       stream, (float*)out, (const float*)input, (long)rows, d,
+                       alpha, limit);
+  else
+    hipLaunchKernelGGL(clamped_swiglu_kernel<short>, dim3(grid), dim3(256), 0,
+                       stream, (short*)out, (const short*)input, (long)rows, d,
+                       alpha, limit);
   HIP_CHECK_KERNEL();
   return hipSuccess;
 }

@@ -1,10 +1,6 @@
 // Python bindings for the CDNA4 kernels (torch extension, ROCm-native:
 // c10::hip stream APIs, no CUDA-compat shims).
-#include <torch/extension.h>
-
-#include <c10/hip/HIPStream.h>
-
-#include <hip/hip_runtime.h>
+#include "bindings_common.h"
 
 // launchers from the .hip translation units
 extern "C" {
@@ -46,12 +42,6 @@ hipError_t ks_fused_add_layer_norm(void*, const void*, const void*,
                                    const void*, const void*, float, int, int,
                                    hipStream_t);
 hipError_t ks_gelu(void*, const void*, long, hipStream_t);
-hipError_t ks_greedy_sample(void*, const void*, int, int, hipStream_t);
-hipError_t ks_gumbel_sample(void*, const void*, const void*, const void*,
-                            const void*, int, int, hipStream_t);
-hipError_t ks_topk_topp_sample(void*, const void*, const void*, const void*,
-                               const void*, const void*, int, int,
-                               hipStream_t);
 hipError_t ks_mfma_probe(void*, const void*, const void*, hipStream_t);
 hipError_t ks_skinny_gemm(void*, void*, const void*, const void*, int, int,
                           int, long, hipStream_t);
@@ -60,20 +50,6 @@ hipError_t ks_gemm8(void*, const void*, const void*, int, int, int, int,
 }
 
 namespace {
-
-hipStream_t current_stream() {
-  return c10::hip::getCurrentHIPStream().stream();
-}
-
-void check_hip(hipError_t err, const char* op) {
-  TORCH_CHECK(err == hipSuccess, op, " failed: ", hipGetErrorString(err));
-}
-
-#define CHECK_BF16_CONTIG(t)                                       \
-  TORCH_CHECK((t).scalar_type() == at::kBFloat16, #t " must be bf16"); \
-  TORCH_CHECK((t).is_contiguous(), #t " must be contiguous");      \
-  TORCH_CHECK((t).is_cuda(), #t " must be on GPU")
-
 // [T, heads, D] where rows may be strided (qkv split views) but the
 // (head, dim) block of each row is dense
 #define CHECK_KV_CACHE(t)                                               \
@@ -335,46 +311,6 @@ void gelu(at::Tensor& out, at::Tensor& input) {
             "gelu");
 }
 
-void greedy_sample(at::Tensor& out, at::Tensor& logits) {
-  CHECK_BF16_CONTIG(logits);
-  TORCH_CHECK(out.scalar_type() == at::kLong, "out int64");
-  check_hip(ks_greedy_sample(out.data_ptr(), logits.data_ptr(),
-                             logits.size(0), logits.size(1),
-                             current_stream()),
-            "greedy_sample");
-}
-
-void gumbel_sample(at::Tensor& out, at::Tensor& logits,
-                   at::Tensor& temperatures, at::Tensor& top_k,
-                   at::Tensor& seeds) {
-  CHECK_BF16_CONTIG(logits);
-  TORCH_CHECK(out.scalar_type() == at::kLong, "out int64");
-  TORCH_CHECK(temperatures.scalar_type() == at::kFloat, "temps fp32");
-  TORCH_CHECK(seeds.scalar_type() == at::kLong, "seeds int64");
-  check_hip(ks_gumbel_sample(out.data_ptr(), logits.data_ptr(),
-                             temperatures.data_ptr(), top_k.data_ptr(),
-                             seeds.data_ptr(), logits.size(0), logits.size(1),
-                             current_stream()),
-            "gumbel_sample");
-}
-
-void topk_topp_sample(at::Tensor& out, at::Tensor& logits,
-                      at::Tensor& temperatures, at::Tensor& top_p,
-                      at::Tensor& top_k, at::Tensor& seeds) {
-  CHECK_BF16_CONTIG(logits);
-  TORCH_CHECK(out.scalar_type() == at::kLong, "out int64");
-  TORCH_CHECK(temperatures.scalar_type() == at::kFloat, "temps fp32");
-  TORCH_CHECK(top_p.scalar_type() == at::kFloat, "top_p fp32");
-  TORCH_CHECK(top_k.scalar_type() == at::kInt, "top_k int32");
-  TORCH_CHECK(seeds.scalar_type() == at::kLong, "seeds int64");
-  check_hip(ks_topk_topp_sample(out.data_ptr(), logits.data_ptr(),
-                                temperatures.data_ptr(), top_p.data_ptr(),
-                                top_k.data_ptr(), seeds.data_ptr(),
-                                logits.size(0), logits.size(1),
-                                current_stream()),
-            "topk_topp_sample");
-}
-
 void skinny_gemm(at::Tensor& out, at::Tensor& x, at::Tensor& w) {
   // out [N, M] bf16 = x [N, K] @ w [M, K]^T  (decode shapes, N <= 256)
   CHECK_BF16_CONTIG(out);
@@ -446,10 +382,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("fused_add_layer_norm", &fused_add_layer_norm,
         "residual-add + LayerNorm");
   m.def("gelu", &gelu, "erf GELU");
-  m.def("greedy_sample", &greedy_sample, "argmax sampling");
-  m.def("gumbel_sample", &gumbel_sample, "Gumbel-max temperature sampling");
-  m.def("topk_topp_sample", &topk_topp_sample,
-        "fused top-k/top-p + Gumbel-max sampler (radix-histogram select)");
+  def_sampling(m);
   m.def("skinny_gemm", &skinny_gemm, "decode GEMM (N<=256, MFMA streaming)");
   m.def("gemm8", &gemm8,
         "EXPERIMENTAL 8-phase 256x256 MFMA GEMM (round-2 candidate)");

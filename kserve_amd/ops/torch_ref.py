@@ -310,3 +310,162 @@ def fused_add_layer_norm(
 
 def gelu(x: torch.Tensor) -> torch.Tensor:
     return torch.nn.functional.gelu(x.float()).to(x.dtype)
+
+
+# ---------------------------------------------------------------------------
+# Mechanisms of models with a 32-bit residual stream and recurrent state.
+# CPU forms of the kernels in residual_norm_f32.hip / ssm_scan.hip /
+# attention_f32.hip; same arguments, same in-place effects on caches/state.
+# ---------------------------------------------------------------------------
+
+
+def sinusoid_inv_freq(width: int, base: float = 10000.0) -> torch.Tensor:
+    """inv_freq[i] = base^(-2i/width), rounded once from float64."""
+    i = torch.arange((width + 1) // 2, dtype=torch.float64)
+    return (base ** (-2.0 * i / width)).to(torch.float32)
+
+
+def embed_scale_sinpos(table, tokens, positions, inv_freq, scale: float):
+    width = table.shape[1]
+    ang = positions.to(torch.float32).unsqueeze(1) * inv_freq.unsqueeze(0)
+    pe = torch.stack([torch.sin(ang), torch.cos(ang)], dim=-1).reshape(
+        tokens.shape[0], -1
+    )[:, :width]
+    return table[tokens].float() * scale + pe
+
+
+def add_rms_norm_f32res(
+    residual, weight, eps, w_offset, out_dtype, d0=None, s0=1.0, d1=None, s1=1.0
+):
+    if d0 is not None:
+        residual += s0 * d0.float()
+    if d1 is not None:
+        residual += s1 * d1.float()
+    inv = torch.rsqrt(residual.pow(2).mean(-1, keepdim=True) + eps)
+    return (residual * inv * (w_offset + weight)).to(out_dtype)
+
+
+def gated_group_rms_norm(y, z, weight, eps, groups: int, out_dtype):
+    zf = z.float()
+    v = y * (zf * torch.sigmoid(zf))
+    vg = v.reshape(v.shape[0], groups, -1)
+    vg = vg * torch.rsqrt(vg.pow(2).mean(-1, keepdim=True) + eps)
+    return (vg.reshape(v.shape) * weight).to(out_dtype)
+
+
+def causal_conv_silu(x_in, w, bias, conv_state, positions, cu_seqlens, slots):
+    taps = w.shape[1]
+    hist = taps - 1
+    out = torch.empty(x_in.shape, dtype=torch.float32)
+    cu = cu_seqlens.tolist()
+    for s, slot in enumerate(slots.tolist()):
+        a, b = cu[s], cu[s + 1]
+        if b <= a:
+            continue
+        start = int(positions[a])
+        prev = conv_state[slot, :hist].float().clone()
+        # history rows hold positions start-hist .. start-1; zeros before 0
+        for i in range(hist):
+            if start - hist + i < 0:
+                prev[i] = 0
+        full = torch.cat([prev, x_in[a:b].float()], dim=0)
+        acc = bias.unsqueeze(0).expand(b - a, -1).clone()
+        for j in range(taps):
+            acc = acc + full[j : j + b - a] * w[:, j].unsqueeze(0)
+        out[a:b] = acc * torch.sigmoid(acc)
+        if hist:
+            conv_state[slot, :hist] = full[full.shape[0] - hist :].to(
+                conv_state.dtype
+            )
+    return out
+
+
+def ssd_scan(
+    xbc, dt_raw, dt_bias, a_log, d_skip, state, positions, cu_seqlens, slots,
+    groups: int,
+):
+    _, heads, P, N = state.shape
+    inner = heads * P
+    T = xbc.shape[0]
+    y = torch.empty(T, inner, dtype=torch.float32)
+    cu = cu_seqlens.tolist()
+    A = -torch.exp(a_log)
+    rep = heads // groups
+    for s, slot in enumerate(slots.tolist()):
+        a, b = cu[s], cu[s + 1]
+        if b <= a:
+            continue
+        S = state[slot].clone()  # [heads, P, N]
+        if int(positions[a]) == 0:
+            S.zero_()
+        for t in range(a, b):
+            x = xbc[t, :inner].reshape(heads, P)
+            B = xbc[t, inner : inner + groups * N].reshape(groups, N)
+            C = xbc[t, inner + groups * N :].reshape(groups, N)
+            B = B.repeat_interleave(rep, dim=0)
+            C = C.repeat_interleave(rep, dim=0)
+            v = dt_raw[t].float() + dt_bias
+            dt = torch.where(v > 30.0, v, torch.log1p(torch.exp(v)))
+            decay = torch.exp(A * dt)
+            S = decay[:, None, None] * S + (dt[:, None] * x)[:, :, None] * B[:, None, :]
+            y[t] = ((S * C[:, None, :]).sum(-1) + d_skip[:, None] * x).reshape(-1)
+        state[slot] = S
+    return y
+
+
+def qk_norm_temp_cache(
+    q, k, v, qw, kw, positions, slot_mapping, k_cache, v_cache, eps,
+    temp_coef: float, temp_every: int, heads: int,
+):
+    _, G, bs, D = k_cache.shape
+    DV = v_cache.shape[3]
+    qf, kf = q.float(), k.float()
+    qn = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps) * qw
+    kn = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps) * kw
+    if temp_every > 0:
+        steps = torch.div(positions + 1, temp_every, rounding_mode="floor")
+        qn = qn * (1.0 + temp_coef * torch.log(steps.float() + 1.0)).unsqueeze(1)
+    slots = slot_mapping.long()
+    ok = slots >= 0
+    blk, off = slots[ok] // bs, slots[ok] % bs
+    k_cache[blk, :, off] = kn[ok].reshape(-1, G, D).to(k_cache.dtype)
+    v_cache[blk, :, off] = v[ok].reshape(-1, G, DV).to(v_cache.dtype)
+    return qn
+
+
+def ctx_attention_f32(
+    q, k_cache, v_cache, block_tables, cu_q, ctx_lens, scale: float,
+    heads: int, gate=None, out_dtype=torch.float32,
+):
+    _, G, bs, D = k_cache.shape
+    DV = v_cache.shape[3]
+    T = q.shape[0]
+    out = torch.zeros(T, heads, DV, dtype=torch.float32)
+    cu = cu_q.tolist()
+    rep = heads // G
+    for s, ctx in enumerate(ctx_lens.tolist()):
+        a, b = cu[s], cu[s + 1]
+        if b <= a:
+            continue
+        nb = -(-ctx // bs)
+        blocks = block_tables[s, :nb].long()
+        K = k_cache[blocks].float().permute(1, 0, 2, 3).reshape(G, nb * bs, D)[:, :ctx]
+        V = v_cache[blocks].float().permute(1, 0, 2, 3).reshape(G, nb * bs, DV)[:, :ctx]
+        K = K.repeat_interleave(rep, dim=0)
+        V = V.repeat_interleave(rep, dim=0)
+        qs = q[a:b].reshape(b - a, heads, D).float().transpose(0, 1)
+        sc = torch.matmul(qs, K.transpose(1, 2)) * scale  # [heads, n, ctx]
+        qpos = torch.arange(ctx - (b - a), ctx).unsqueeze(1)
+        vis = torch.arange(ctx).unsqueeze(0) <= qpos
+        sc = sc.masked_fill(~vis.unsqueeze(0), float("-inf"))
+        out[a:b] = torch.matmul(torch.softmax(sc, dim=-1), V).transpose(0, 1)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float()).unsqueeze(-1)
+    return out.reshape(T, heads * DV).to(out_dtype)
+
+
+def clamped_swiglu(x, alpha: float, limit: float):
+    d = x.shape[-1] // 2
+    g = x[..., :d].float().clamp(max=limit)
+    u = x[..., d:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(x.dtype)
