@@ -57,6 +57,10 @@ class ModelRunner:
         # pinned staging + per-request numpy block-table cache
         self._pin: Optional[Dict[str, torch.Tensor]] = None
         self._pin_np = None
+        # recorded after a step's async copies out of the pinned buffers; the
+        # next fill waits on it, so a caller that never reads the step's
+        # result back cannot overwrite inputs still in flight
+        self._pin_event = None
         self._bt_cache: Dict[str, object] = {}
         # host-DRAM KV offload tier (pinned) + dedicated copy stream
         self.cpu_kv_caches: List[Tuple[torch.Tensor, torch.Tensor]] = []
@@ -374,6 +378,7 @@ class ModelRunner:
         (n, nb) = batch size and max block-table width used."""
         import numpy as np
 
+        self._wait_staging()
         n = len(batch.requests)
         bs = self.config.cache.block_size
         max_blocks = 1
@@ -409,6 +414,16 @@ class ModelRunner:
             btab[i, : cache[1].shape[0]] = cache[1]
         return n, max_blocks
 
+    def _wait_staging(self) -> None:
+        if self._pin_event is not None:
+            self._pin_event.synchronize()
+            self._pin_event = None
+
+    def _mark_staging(self) -> None:
+        if self.is_cuda:
+            self._pin_event = torch.cuda.Event()
+            self._pin_event.record(torch.cuda.current_stream())
+
     def release_request(self, request_id: str):
         self._bt_cache.pop(request_id, None)
 
@@ -431,6 +446,7 @@ class ModelRunner:
             )
         input_ids = pin["input_ids"][:n].to(dev, non_blocking=True)
         pos = pin["positions"][:n].to(dev, non_blocking=True)
+        self._mark_staging()
         return input_ids, pos, meta
 
     def _decode_layout_meta(self, meta, n: int, state_slots) -> None:
@@ -720,6 +736,7 @@ class ModelRunner:
         buf["block_tables"][:bucket, :nb].copy_(
             pin["block_tables"][:bucket, :nb], non_blocking=True
         )
+        self._mark_staging()
         self._graphs[bucket].replay()
         return buf["logits"][bucket][:n]
 
@@ -745,6 +762,7 @@ class ModelRunner:
         buf["block_tables"][:bucket, :nb].copy_(
             pin["block_tables"][:bucket, :nb], non_blocking=True
         )
+        self._mark_staging()
         return n
 
     def _stage_sampling_params(self, bucket: int, requests) -> None:
