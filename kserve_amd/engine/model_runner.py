@@ -25,6 +25,9 @@ _DEFAULT_GRAPH_BATCH_SIZES = [1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256,
 
 
 class ModelRunner:
+    # event after the last async copies out of the pinned staging buffers
+    _pin_event = None
+
     def __init__(
         self,
         config: EngineConfig,
@@ -394,10 +397,11 @@ class ModelRunner:
         sm = pnp["slot_mapping"]
         ctx = pnp["context_lens"]
         btab = pnp["block_tables"]
-        ss = pnp["state_slots"]
+        ss = pnp.get("state_slots")
         for i, req in enumerate(batch.requests):
             pos = req.num_computed_tokens
-            ss[i] = req.state_slot
+            if ss is not None:
+                ss[i] = req.state_slot
             ii[i] = req.all_token_ids[pos]
             pp[i] = pos
             t = tables[i]
