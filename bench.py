@@ -28,6 +28,146 @@ if os.path.exists(_TUNE_BASE.replace(".csv", "0.csv")):
     os.environ.setdefault("PYTORCH_TUNABLEOP_FILENAME", _TUNE_BASE)
 
 
+# layer shapes for --hybrid-compare: widths, head counts and feed-forward
+# sizes of common 1-3B and 7-8B models; the state-space sublayers use the
+# usual 2x inner width, 64-wide heads and 128 states
+HYBRID_SIZES = {
+    "2k": dict(width=2048, heads=16, kv_heads=4, head_dim=128, ff=8192,
+               ssm_heads=64, ssm_vdim=64, state=128, groups=8, vocab=32000),
+    "4k": dict(width=4096, heads=32, kv_heads=8, head_dim=128, ff=14336,
+               ssm_heads=128, ssm_vdim=64, state=128, groups=8, vocab=32000),
+}
+
+
+def _hybrid_model_configs(size: dict, layers: int):
+    from kserve_amd.engine.config import (
+        AttentionMixerSpec,
+        GLUSpec,
+        HybridLayerSpec,
+        HybridModelConfig,
+        ModelConfig,
+        SSMMixerSpec,
+    )
+
+    ssm = SSMMixerSpec(heads=size["ssm_heads"], vdim=size["ssm_vdim"],
+                       state=size["state"], groups=size["groups"], conv=4,
+                       norm_groups=size["groups"])
+    attn = AttentionMixerSpec(heads=size["heads"], kv_heads=size["kv_heads"],
+                              dim=size["head_dim"], vdim=size["head_dim"],
+                              scale=size["head_dim"] ** -0.5,
+                              q_temp_coef=0.1, q_temp_every=1024)
+    mlp = GLUSpec(ff=size["ff"], limit=7.0)
+    specs = []
+    for i in range(layers):
+        if i % 2 == 0:
+            specs.append(HybridLayerSpec("mamba2", ssm=ssm, mlp=mlp))
+        else:
+            specs.append(HybridLayerSpec("parallel", attention=attn, ssm=ssm,
+                                         mlp=mlp))
+    hybrid = HybridModelConfig(vocab_size=size["vocab"],
+                               hidden_size=size["width"], layers=specs,
+                               model_name="merulorn-bench")
+    llama = ModelConfig(vocab_size=size["vocab"], hidden_size=size["width"],
+                        intermediate_size=size["ff"], num_layers=layers,
+                        num_heads=size["heads"], num_kv_heads=size["kv_heads"],
+                        head_dim=size["head_dim"],
+                        max_position_embeddings=8192, model_name="llama-bench")
+    return hybrid, llama
+
+
+def _throughput(mcfg, prompt_len, n_prompts, concurrency, steps, warmup, eager):
+    """(prefill tok/s, decode tok/s) through the engine's own step()."""
+    import torch
+
+    from kserve_amd.engine.config import CacheConfig, EngineConfig, SchedulerConfig
+    from kserve_amd.engine.engine import LLMEngine
+    from kserve_amd.engine.sampling_params import SamplingParams
+
+    window = 8
+    max_len = prompt_len + (steps + warmup + 2) * window + 64
+    blocks = (max(n_prompts, concurrency) + 2) * (-(-max_len // 16)) + 64
+    cfg = EngineConfig(
+        model=mcfg,
+        cache=CacheConfig(block_size=16, num_gpu_blocks=blocks),
+        scheduler=SchedulerConfig(
+            max_num_seqs=max(n_prompts, concurrency),
+            max_num_batched_tokens=n_prompts * prompt_len,
+            max_model_len=max_len, multi_step=window,
+        ),
+        device="cuda", seed=7, enforce_eager=eager, eos_token_id=-1,
+    )
+    engine = LLMEngine(cfg)
+    gen = torch.Generator().manual_seed(3)
+    sp = SamplingParams(temperature=0.0, max_tokens=max_len, ignore_eos=True)
+
+    def submit(n, tag):
+        for i in range(n):
+            engine.add_request(
+                torch.randint(0, mcfg.vocab_size, (prompt_len,), generator=gen).tolist(),
+                sp, request_id=f"{tag}-{i}",
+            )
+
+    # prefill: one step takes n_prompts whole prompts; time the second wave
+    submit(n_prompts, "warm")
+    engine.step()
+    for r in list(engine.scheduler.running):
+        engine.abort_request(r.request_id)
+    submit(n_prompts, "timed")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    engine.step()
+    torch.cuda.synchronize()
+    prefill = n_prompts * prompt_len / (time.perf_counter() - t0)
+    for r in list(engine.scheduler.running):
+        engine.abort_request(r.request_id)
+
+    # decode: `concurrency` sequences with prompt_len context each
+    submit(concurrency, "dec")
+    while engine.scheduler.num_waiting > 0:
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    tokens = 0
+    for _ in range(steps):
+        tokens += sum(len(o.new_token_ids) for o in engine.step())
+    torch.cuda.synchronize()
+    decode = tokens / (time.perf_counter() - t0)
+    del engine
+    torch.cuda.empty_cache()
+    return prefill, decode
+
+
+def hybrid_compare(args):
+    """Prefill and decode tok/s of the Merulorn design next to a llama model
+    of equal size, both through LLMEngine.step() on one GPU, bf16, random
+    weights. Prints one JSON line per (size, model)."""
+    import torch
+
+    assert torch.cuda.is_available(), "--hybrid-compare needs a GPU"
+    for name in args.hybrid_compare.split(","):
+        size = HYBRID_SIZES[name]
+        hybrid, llama = _hybrid_model_configs(size, layers=4)
+        for label, mcfg in (("hybrid", hybrid), ("llama", llama)):
+            if args.hybrid_only and args.hybrid_only != label:
+                continue
+            prefill, decode = _throughput(
+                mcfg, prompt_len=args.prompt_len if args.prompt_len != 512 else 2048,
+                n_prompts=8, concurrency=min(args.concurrency, 256),
+                steps=args.steps, warmup=args.warmup, eager=args.eager,
+            )
+            print(json.dumps({
+                "bench": "hybrid-compare", "size": name, "model": mcfg.model_name,
+                "layers": 4, "width": size["width"],
+                "prefill_tok_s": round(prefill, 1),
+                "decode_tok_s": round(decode, 1),
+                "prefill_batch": "8 x prompt", "decode_concurrency":
+                    min(args.concurrency, 256),
+                "dtype": "bfloat16", "data": "synthetic, random-init weights",
+            }), flush=True)
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -55,9 +195,22 @@ def main():
                         choices=["auto", "fp8"],
                         help="opt-in fp8 E4M3 KV cache (NOT the headline "
                              "config; bf16 compute is unchanged)")
+    parser.add_argument("--hybrid-compare", type=str, default=None,
+                        metavar="SIZE[,SIZE...]",
+                        help="instead of the flagship workload: prefill and "
+                             "decode throughput of a Merulorn-design model "
+                             "beside a llama model of equal width, heads, "
+                             "feed-forward and depth (sizes: "
+                             + ", ".join(HYBRID_SIZES) + ")")
+    parser.add_argument("--hybrid-only", type=str, default=None,
+                        choices=["hybrid", "llama"],
+                        help="with --hybrid-compare: run one side only "
+                             "(e.g. under a profiler)")
     parser.add_argument("--profile-cpu", action="store_true",
                         help="cProfile the timed loop and print hot functions")
     args = parser.parse_args()
+    if args.hybrid_compare:
+        return hybrid_compare(args)
 
     import torch
 

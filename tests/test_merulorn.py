@@ -90,7 +90,8 @@ def rel_err(got, want):
 
 
 def tol(backend):
-    return 4e-2 if backend[1] == "bfloat16" else 2e-4
+    # bf16: worst position of a few hundred, inputs and products rounded
+    return 6e-2 if backend[1] == "bfloat16" else 2e-4
 
 
 def run_schedule(engine, prompts, schedule):
@@ -319,7 +320,7 @@ class TestFarKeys:
         plain = list(toks)
         plain[page_pos] = 3
         # the needle matters: without it the last logits move visibly
-        assert rel_err(O.forward(cfg, sd, plain)[-1:], want[-1:]) > 20 * tol(backend)
+        assert rel_err(O.forward(cfg, sd, plain)[-1:], want[-1:]) > 0.2
         eng = make_engine(cfg, sd, backend, num_blocks=32)
         got = run_schedule(eng, [toks], [[(0, 150)]] + [[(0, 1)]] * 50)[0]
         assert rel_err(got, want) < tol(backend)

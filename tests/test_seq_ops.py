@@ -349,4 +349,4 @@ class TestAttention:
         want = torch.softmax(sc, 0) @ v.to(be[1]).double()
         close(out[0, :DV], want, be)
         close(out[0, DV:], want, be)
-        assert (want - v[3].double()).abs().max() < 1e-3
+        assert (want - v.to(be[1])[3].double()).abs().max() < 1e-3
