@@ -8,24 +8,32 @@
 //    write q (fp32) out and scatter k / v into the paged cache.
 //  * ctx_attention_f32: causal attention of a flat variable-length query
 //    batch against each sequence's pages (the portion's own keys are already
-//    in the cache). Queries of one block share a kv head: in prefill a block
-//    takes 16 consecutive tokens of one query head, in decode it takes the
-//    query heads of one group so the group's K/V tile is staged once.
-//    K/V tiles of 64 keys are converted to fp32 in LDS; a lane owns one key
-//    for the score and softmax phase and one output column per 64 for the
-//    weighted sum. An optional per-(token, head) gate multiplies the result
-//    by sigmoid(gate) before it is stored.
+//    in the cache). Both products run on the fp32 matrix cores
+//    (v_mfma_f32_16x16x4_f32), so q.k, the softmax weights and weights x V
+//    are all true fp32 whatever the cache dtype; K/V tiles of 64 keys are
+//    converted to fp32 while they are staged in LDS.
+//    The kernel works on transposed tiles: S^T = K Q^T puts one query per
+//    lane column, so the running max / sum / rescale are per-lane scalars,
+//    and the S^T accumulator registers are already the B operand of
+//    O^T += V^T P^T (the contraction runs over keys in the accumulator's own
+//    order; V is read from LDS in that order), so the weights never leave
+//    registers.
+//    Prefill: a block takes 64 consecutive tokens of one query head, 16 per
+//    wave, all waves sharing the staged K/V tile. Decode (one token per
+//    sequence): a block takes the query heads of one KV group as its 16
+//    columns and the four waves split every tile's keys, merging their
+//    partial (max, sum, O) through LDS at the end, so the group's K/V is read
+//    once. Head sizes are padded up to 64/128/256 with zeros. An optional
+//    per-(token, head) gate multiplies the result by sigmoid(gate).
 #include "dtype_io.h"
 
 namespace {
 
 constexpr int NT = 256;
 constexpr int NW = NT / WAVE_SIZE;
-constexpr int ROWS = 16;          // query rows per block
-constexpr int RPW = ROWS / NW;    // rows per wave
-constexpr int BK = 64;            // keys per tile (lane <-> key)
-constexpr int MAX_DV = 256;
-constexpr int NVC = MAX_DV / 64;  // output columns per lane
+constexpr int BK = 64;  // keys per staged tile
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 template <typename T>
 __global__ void qk_norm_temp_cache_kernel(
@@ -75,7 +83,67 @@ __global__ void qk_norm_temp_cache_kernel(
   }
 }
 
+// 8 consecutive elements of a cache row -> fp32
 template <typename T>
+__device__ __forceinline__ void load8(const T* p, bool vec, int valid, float* v);
+template <>
+__device__ __forceinline__ void load8<short>(const short* p, bool vec, int valid,
+                                             float* v) {
+  if (vec && valid >= 8) {
+    const short8_t x = *reinterpret_cast<const short8_t*>(p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = bf16_bits_to_float(x[i]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = i < valid ? bf16_bits_to_float(p[i]) : 0.f;
+  }
+}
+template <>
+__device__ __forceinline__ void load8<float>(const float* p, bool vec, int valid,
+                                             float* v) {
+  if (vec && valid >= 8) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[i] = a[i];
+      v[4 + i] = b[i];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = i < valid ? p[i] : 0.f;
+  }
+}
+
+// stage rows [k0, k0 + nk) of one kv head into LDS as fp32 [BK][WP + 4],
+// zero-filled past the head size and past nk
+template <typename T, int WP>
+__device__ __forceinline__ void stage_tile(float* dst, const T* cache,
+                                           const int* bt, int k0, int nk, int g,
+                                           int kv_heads, int W, int block_size,
+                                           bool vec) {
+  constexpr int CPR = WP / 8;  // 8-element chunks per row
+  constexpr int LS = WP + 4;
+  for (int c = threadIdx.x; c < BK * CPR; c += NT) {
+    const int j = c / CPR, d0 = (c % CPR) * 8;
+    float v[8];
+    const int valid = j < nk ? W - d0 : 0;
+    if (valid > 0) {
+      const int kp = k0 + j;
+      const long blk = bt[kp / block_size];
+      load8<T>(cache + ((blk * kv_heads + g) * block_size + kp % block_size) * W + d0,
+               vec, valid, v);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = 0.f;
+    }
+    f32x4* o = reinterpret_cast<f32x4*>(dst + j * LS + d0);
+    o[0] = f32x4{v[0], v[1], v[2], v[3]};
+    o[1] = f32x4{v[4], v[5], v[6], v[7]};
+  }
+}
+
+template <typename T, int DP, int DVP, bool SPLITK>
 __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     T* __restrict__ out, const float* __restrict__ q,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -84,6 +152,12 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     const T* __restrict__ gate, long gate_stride, float scale, int heads,
     int kv_heads, int D, int DV, int block_size, int hpb) {
   extern __shared__ float lds[];
+  constexpr int KS = DP + 4;   // K row stride: lanes of one MFMA read hit 64 banks
+  constexpr int VS = DVP + 4;  // V row stride: likewise for the 4-key-apart rows
+  constexpr int ROWS = SPLITK ? 16 : 64;  // query rows per block
+  float* Ks = lds;             // [BK][KS]
+  float* Vs = Ks + BK * KS;    // [BK][VS]
+
   const int s = blockIdx.y;
   const int q0 = cu_q[s];
   const int q_len = cu_q[s + 1] - q0;
@@ -95,132 +169,161 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   const int ctx = ctx_lens[s];
   const int ntok = min(tpb, q_len - tok0);
   const int nrows = ntok * hpb;
-  // absolute position of the block's last query bounds the keys it needs
-  const int last_pos = ctx - q_len + tok0 + ntok - 1;
-
-  const int KS = D + 1;  // padded K row: lane-per-key reads hit distinct banks
-  float* Ks = lds;                   // [BK][D+1]
-  float* Vs = Ks + BK * KS;          // [BK][DV]
-  float* Qs = Vs + BK * DV;          // [D][ROWS] (transposed)
-  float* Ps = Qs + D * ROWS;         // [NW][BK][RPW]
+  const int base_pos = ctx - q_len + tok0;  // position of the block's first token
+  const int last_pos = base_pos + ntok - 1;
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
+  const int li = lane & 15;  // query column of this lane
+  const int lg = lane >> 4;
 
-  // stage the block's queries, pre-multiplied by the softmax scale
-  for (int e = threadIdx.x; e < ROWS * D; e += NT) {
-    const int r = e / D, d = e % D;
-    float v = 0.f;
-    if (r < nrows) {
-      const int tok = q0 + tok0 + r / hpb, hd = head0 + r % hpb;
-      v = q[((long)tok * heads + hd) * D + d] * scale;
-    }
-    Qs[d * ROWS + r] = v;
-  }
+  // this lane's query
+  const int r = (SPLITK ? 0 : wave * 16) + li;
+  const bool row_ok = r < nrows;
+  const int tok = q0 + tok0 + r / hpb;
+  const int hd = head0 + r % hpb;
+  const int qpos = row_ok ? base_pos + r / hpb : -1;
+  // keys this wave needs: up to its own last row's position
+  const int wave_last =
+      SPLITK ? last_pos : base_pos + min(wave * 16 + 15, nrows - 1) / hpb;
 
-  float m[RPW], l[RPW], acc[RPW][NVC];
-  int qpos[RPW];
+  // Q^T fragments (B operand): lane (k = lg, column li) of k-step ks holds
+  // q[query li][4 ks + lg], pre-multiplied by the softmax scale
+  float qf[DP / 4];
 #pragma unroll
-  for (int i = 0; i < RPW; ++i) {
-    m[i] = -INFINITY;
-    l[i] = 0.f;
-    const int r = wave * RPW + i;
-    qpos[i] = r < nrows ? ctx - q_len + tok0 + r / hpb : -1;
-#pragma unroll
-    for (int c = 0; c < NVC; ++c) acc[i][c] = 0.f;
+  for (int ks = 0; ks < DP / 4; ++ks) {
+    const int d = 4 * ks + lg;
+    qf[ks] = (row_ok && d < D) ? q[((long)tok * heads + hd) * D + d] * scale : 0.f;
   }
+  f32x4 o[DVP / 16];
+#pragma unroll
+  for (int i = 0; i < DVP / 16; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
   const int* bt = block_tables + (long)s * bt_stride;
+  const bool kvec = (D % 8) == 0, vvec = (DV % 8) == 0;
+  constexpr int KT = SPLITK ? 1 : 4;  // 16-key sub-tiles per wave and tile
 
   for (int k0 = 0; k0 <= last_pos; k0 += BK) {
-    __syncthreads();  // previous tile fully consumed (and Qs visible)
+    __syncthreads();  // previous tile fully consumed
     const int nk = min(BK, last_pos + 1 - k0);
-    for (int e = threadIdx.x; e < BK * D; e += NT) {
-      const int j = e / D, d = e % D;
-      float v = 0.f;
-      if (j < nk) {
-        const int kp = k0 + j;
-        const long blk = bt[kp / block_size];
-        v = ld_f32(k_cache,
-                   ((blk * kv_heads + g) * block_size + kp % block_size) * D + d);
-      }
-      Ks[j * KS + d] = v;
-    }
-    for (int e = threadIdx.x; e < BK * DV; e += NT) {
-      const int j = e / DV, d = e % DV;
-      float v = 0.f;
-      if (j < nk) {
-        const int kp = k0 + j;
-        const long blk = bt[kp / block_size];
-        v = ld_f32(v_cache,
-                   ((blk * kv_heads + g) * block_size + kp % block_size) * DV + d);
-      }
-      Vs[j * DV + d] = v;
-    }
+    stage_tile<T, DP>(Ks, k_cache, bt, k0, nk, g, kv_heads, D, block_size, kvec);
+    stage_tile<T, DVP>(Vs, v_cache, bt, k0, nk, g, kv_heads, DV, block_size, vvec);
     __syncthreads();
+    if (k0 > wave_last) continue;
 
-    // scores: lane = key, RPW rows of this wave at once
-    float sc[RPW];
+    // S^T sub-tiles: acc[kt][v] = score(key k0 + 16 kt' + 4 lg + v, query li)
+    f32x4 sc[KT];
 #pragma unroll
-    for (int i = 0; i < RPW; ++i) sc[i] = 0.f;
-    const float* krow = Ks + lane * KS;
-    const float* qcol = Qs + wave * RPW;
-    for (int d = 0; d < D; ++d) {
-      const float kv = krow[d];
+    for (int t = 0; t < KT; ++t) {
+      const int kt = SPLITK ? wave : t;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      const float* ka = Ks + (16 * kt + li) * KS + lg;
 #pragma unroll
-      for (int i = 0; i < RPW; ++i) sc[i] += qcol[d * ROWS + i] * kv;
+      for (int ks = 0; ks < DP / 4; ++ks)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[4 * ks], qf[ks], acc, 0, 0, 0);
+      sc[t] = acc;
     }
-    const int kp = k0 + lane;
-    float* pw = Ps + wave * BK * RPW;
+    float mt = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < RPW; ++i) {
-      const bool vis = kp <= qpos[i];
-      const float sv = vis ? sc[i] : -INFINITY;
-      const float mt = wave_reduce_max(sv);
-      const float mn = fmaxf(m[i], mt);
-      // a row with no visible key in this tile keeps mn = -inf only while
-      // it has seen nothing at all; guard the exp arguments
-      const float corr = (mn == -INFINITY) ? 1.f : expf(m[i] - mn);
-      const float pv = vis ? expf(sv - mn) : 0.f;
-      l[i] = l[i] * corr + wave_reduce_sum(pv);
-      m[i] = mn;
+    for (int t = 0; t < KT; ++t) {
+      const int kt = SPLITK ? wave : t;
 #pragma unroll
-      for (int c = 0; c < NVC; ++c) acc[i][c] *= corr;
-      pw[lane * RPW + i] = pv;
+      for (int v = 0; v < 4; ++v) {
+        const int kp = k0 + 16 * kt + 4 * lg + v;
+        sc[t][v] = kp <= qpos ? sc[t][v] : -INFINITY;
+        mt = fmaxf(mt, sc[t][v]);
+      }
     }
-    // weighted sum: lane = output column (+64 c); weights broadcast from LDS
-    // (each wave reads only what it wrote: no block barrier needed)
-    for (int j = 0; j < nk; ++j) {
-      float pj[RPW];
+    mt = fmaxf(mt, __shfl_xor(mt, 16, WAVE_SIZE));
+    mt = fmaxf(mt, __shfl_xor(mt, 32, WAVE_SIZE));
+    const float mn = fmaxf(m, mt);
+    // a column that has seen no visible key yet keeps mn = -inf
+    const float corr = (mn == -INFINITY) ? 1.f : expf(m - mn);
+    float ps = 0.f;
 #pragma unroll
-      for (int i = 0; i < RPW; ++i) pj[i] = pw[j * RPW + i];
+    for (int t = 0; t < KT; ++t)
 #pragma unroll
-      for (int c = 0; c < NVC; ++c) {
-        const int col = lane + 64 * c;
-        if (col < DV) {
-          const float vv = Vs[j * DV + col];
+      for (int v = 0; v < 4; ++v) {
+        const float pv = sc[t][v] == -INFINITY ? 0.f : expf(sc[t][v] - mn);
+        sc[t][v] = pv;
+        ps += pv;
+      }
+    ps += __shfl_xor(ps, 16, WAVE_SIZE);
+    ps += __shfl_xor(ps, 32, WAVE_SIZE);
+    l = l * corr + ps;
+    m = mn;
 #pragma unroll
-          for (int i = 0; i < RPW; ++i) acc[i][c] += pj[i] * vv;
-        }
+    for (int i = 0; i < DVP / 16; ++i) o[i] *= corr;
+    // O^T += V^T P^T, contraction index of k-step v = key 4 lg + v
+#pragma unroll
+    for (int t = 0; t < KT; ++t) {
+      const int kt = SPLITK ? wave : t;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const float* va = Vs + (16 * kt + 4 * lg + v) * VS + li;
+        const float pb = sc[t][v];
+#pragma unroll
+        for (int i = 0; i < DVP / 16; ++i)
+          o[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(va[16 * i], pb, o[i], 0, 0, 0);
       }
     }
   }
 
-#pragma unroll
-  for (int i = 0; i < RPW; ++i) {
-    const int r = wave * RPW + i;
-    if (r >= nrows) continue;
-    const int tok = q0 + tok0 + r / hpb, hd = head0 + r % hpb;
-    float f = 1.0f / l[i];
-    if (gate) {
-      const float gv = ld_f32(gate, (long)tok * gate_stride + hd);
-      f *= 1.0f / (1.0f + expf(-gv));
+  if (SPLITK) {
+    // merge the four waves' partial results: Ms/Ls [NW][16], Os [NW][16][DVP]
+    __syncthreads();
+    float* Ms = lds;
+    float* Ls = Ms + NW * 16;
+    float* Os = Ls + NW * 16;
+    if (lg == 0) {
+      Ms[wave * 16 + li] = m;
+      Ls[wave * 16 + li] = l;
     }
 #pragma unroll
-    for (int c = 0; c < NVC; ++c) {
-      const int col = lane + 64 * c;
-      if (col < DV) st_f32(out, ((long)tok * heads + hd) * DV + col, acc[i][c] * f);
+    for (int i = 0; i < DVP / 16; ++i)
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        Os[(wave * 16 + li) * DVP + 16 * i + 4 * lg + v] = o[i][v];
+    __syncthreads();
+    for (int e = threadIdx.x; e < nrows * DVP; e += NT) {
+      const int row = e / DVP, dv = e % DVP;
+      if (dv >= DV) continue;
+      float M = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) M = fmaxf(M, Ms[w * 16 + row]);
+      float L = 0.f, O = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const float mw = Ms[w * 16 + row];
+        const float f = mw == -INFINITY ? 0.f : expf(mw - M);
+        L += Ls[w * 16 + row] * f;
+        O += Os[(w * 16 + row) * DVP + dv] * f;
+      }
+      const int tk = q0 + tok0 + row / hpb, h2 = head0 + row % hpb;
+      float f = 1.0f / L;
+      if (gate) {
+        const float gv = ld_f32(gate, (long)tk * gate_stride + h2);
+        f *= 1.0f / (1.0f + expf(-gv));
+      }
+      st_f32(out, ((long)tk * heads + h2) * DV + dv, O * f);
     }
+    return;
   }
+
+  if (!row_ok) return;
+  float f = 1.0f / l;
+  if (gate) {
+    const float gv = ld_f32(gate, (long)tok * gate_stride + hd);
+    f *= 1.0f / (1.0f + expf(-gv));
+  }
+#pragma unroll
+  for (int i = 0; i < DVP / 16; ++i)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int dv = 16 * i + 4 * lg + v;
+      if (dv < DV) st_f32(out, ((long)tok * heads + hd) * DV + dv, o[i][v] * f);
+    }
 }
 
 }  // namespace
@@ -252,6 +355,71 @@ extern "C" hipError_t ks_qk_norm_temp_cache(
   return hipSuccess;
 }
 
+template <typename T, int DP, int DVP>
+hipError_t launch_ctx_attention(void* out, const void* q, const void* k_cache,
+                                const void* v_cache, const void* block_tables,
+                                int bt_stride, const void* cu_q,
+                                const void* ctx_lens, const void* gate,
+                                long gate_stride, float scale, int num_seqs,
+                                int max_q_len, int heads, int kv_heads, int D,
+                                int DV, int block_size, hipStream_t stream) {
+  size_t smem = sizeof(float) * (size_t)BK * (DP + 4 + DVP + 4);
+  const bool decode = max_q_len == 1;
+  // decode: one token per sequence, a block takes heads of one group
+  int hpb = 1;
+  if (decode) {
+    const int gs = heads / kv_heads;
+    for (int c = 1; c <= 16 && c <= gs; ++c)
+      if (gs % c == 0) hpb = c;
+    const size_t merge = sizeof(float) * (size_t)NW * 16 * (DVP + 2);
+    if (merge > smem) smem = merge;
+  }
+  const int rows = decode ? 16 : 64;
+  dim3 grid(cdiv(max_q_len, rows / hpb), num_seqs, heads / hpb);
+  auto fn = decode ? ctx_attention_f32_kernel<T, DP, DVP, true>
+                   : ctx_attention_f32_kernel<T, DP, DVP, false>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(
+        (const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(fn, grid, dim3(NT), smem, stream, (T*)out, (const float*)q,
+                     (const T*)k_cache, (const T*)v_cache,
+                     (const int*)block_tables, bt_stride, (const int*)cu_q,
+                     (const int*)ctx_lens, (const T*)gate, gate_stride, scale,
+                     heads, kv_heads, D, DV, block_size, hpb);
+  return hipGetLastError();
+}
+
+#define CTX_ARGS                                                              \
+  out, q, k_cache, v_cache, block_tables, bt_stride, cu_q, ctx_lens, gate,    \
+      gate_stride, scale, num_seqs, max_q_len, heads, kv_heads, D, DV,        \
+      block_size, stream
+
+template <typename T, int DP>
+hipError_t dispatch_dv(void* out, const void* q, const void* k_cache,
+                       const void* v_cache, const void* block_tables,
+                       int bt_stride, const void* cu_q, const void* ctx_lens,
+                       const void* gate, long gate_stride, float scale,
+                       int num_seqs, int max_q_len, int heads, int kv_heads,
+                       int D, int DV, int block_size, hipStream_t stream) {
+  if (DV <= 64) return launch_ctx_attention<T, DP, 64>(CTX_ARGS);
+  if (DV <= 128) return launch_ctx_attention<T, DP, 128>(CTX_ARGS);
+  return launch_ctx_attention<T, DP, 256>(CTX_ARGS);
+}
+
+template <typename T>
+hipError_t dispatch_d(void* out, const void* q, const void* k_cache,
+                      const void* v_cache, const void* block_tables,
+                      int bt_stride, const void* cu_q, const void* ctx_lens,
+                      const void* gate, long gate_stride, float scale,
+                      int num_seqs, int max_q_len, int heads, int kv_heads,
+                      int D, int DV, int block_size, hipStream_t stream) {
+  if (D <= 64) return dispatch_dv<T, 64>(CTX_ARGS);
+  if (D <= 128) return dispatch_dv<T, 128>(CTX_ARGS);
+  return dispatch_dv<T, 256>(CTX_ARGS);
+}
+
 extern "C" hipError_t ks_ctx_attention_f32(
     void* out, const void* q, const void* k_cache, const void* v_cache,
     const void* block_tables, int bt_stride, const void* cu_q,
@@ -259,51 +427,8 @@ extern "C" hipError_t ks_ctx_attention_f32(
     int num_seqs, int max_q_len, int heads, int kv_heads, int D, int DV,
     int block_size, int is_f32, hipStream_t stream) {
   if (num_seqs == 0 || max_q_len == 0) return hipSuccess;
-  if (DV > MAX_DV || D < 1 || kv_heads < 1 || heads % kv_heads != 0)
+  if (D < 1 || D > 256 || DV < 1 || DV > 256 || kv_heads < 1 ||
+      heads % kv_heads != 0)
     return hipErrorInvalidValue;
-  // decode: one token per sequence, so a block takes heads of one group
-  int hpb = 1;
-  if (max_q_len == 1) {
-    const int gs = heads / kv_heads;
-    for (int c = 1; c <= ROWS && c <= gs; ++c)
-      if (gs % c == 0) hpb = c;
-  }
-  const int tpb = ROWS / hpb;
-  const size_t smem =
-      sizeof(float) * ((size_t)BK * (D + 1) + (size_t)BK * DV +
-                       (size_t)D * ROWS + (size_t)NW * BK * RPW);
-  if (smem > 160 * 1024) return hipErrorInvalidValue;
-  dim3 grid(cdiv(max_q_len, tpb), num_seqs, heads / hpb);
-  hipError_t e;
-  if (is_f32) {
-    auto fn = ctx_attention_f32_kernel<float>;
-    if (smem > 48 * 1024) {
-      e = hipFuncSetAttribute((const void*)fn,
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)smem);
-      if (e != hipSuccess) return e;
-    }
-    hipLaunchKernelGGL(fn, grid, dim3(NT), smem, stream, (float*)out,
-                       (const float*)q, (const float*)k_cache,
-                       (const float*)v_cache, (const int*)block_tables,
-                       bt_stride, (const int*)cu_q, (const int*)ctx_lens,
-                       (const float*)gate, gate_stride, scale, heads, kv_heads,
-                       D, DV, block_size, hpb);
-  } else {
-    auto fn = ctx_attention_f32_kernel<short>;
-    if (smem > 48 * 1024) {
-      e = hipFuncSetAttribute((const void*)fn,
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)smem);
-      if (e != hipSuccess) return e;
-    }
-    hipLaunchKernelGGL(fn, grid, dim3(NT), smem, stream, (short*)out,
-                       (const float*)q, (const short*)k_cache,
-                       (const short*)v_cache, (const int*)block_tables,
-                       bt_stride, (const int*)cu_q, (const int*)ctx_lens,
-                       (const short*)gate, gate_stride, scale, heads, kv_heads,
-                       D, DV, block_size, hpb);
-  }
-  HIP_CHECK_KERNEL();
-  return hipSuccess;
+  return is_f32 ? dispatch_d<float>(CTX_ARGS) : dispatch_d<short>(CTX_ARGS);
 }

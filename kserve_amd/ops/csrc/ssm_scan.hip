@@ -16,11 +16,11 @@
 //        a_t = exp(-exp(A_log_h) * dt_t),  dt_t = softplus(dt_raw + dt_bias_h)
 //        S_t = a_t S_{t-1} + dt_t B_t x_t^T        (S: N x P, fp32)
 //        y_t = S_t^T C_t + D_h x_t
-//    The state lives in registers: lane (ns, p) owns rows n = ns + 16 r of
-//    column p, a 16-lane shuffle tree sums the C-contraction. Tokens of a
-//    sequence are walked in order with the next token's operands in flight.
-//    Serves prefill portions and single-token decode alike (grid = sequences
-//    x heads x column tiles, so decode batches fill the chip).
+//    The state lives in registers: lane (ns, pl) owns rows n = ns + 16 r of
+//    a few columns of one head, a 16-lane shuffle tree sums the C-contraction.
+//    Tokens of a sequence are walked in order, a chunk at a time through LDS.
+//    Serves prefill portions and single-token decode alike (grid = column
+//    tiles x heads x sequences, so decode batches fill the chip).
 #include "dtype_io.h"
 
 namespace {
@@ -95,8 +95,15 @@ __global__ void conv_state_update_kernel(
     conv_state[(slot * hist + i) * channels + c] = keep[i];
 }
 
-// R = state rows per lane (N <= 16 R); blockDim = 256 = 16 ns-lanes x 16 cols
-template <int R>
+// R = state rows per lane (N <= 16 R), PC = columns per lane (tile of 16 PC
+// columns of one head per block). blockDim = 256 = 16 row-lanes x 16 col-lanes.
+// Tokens are taken in chunks of `tc`: the chunk's B, C, x rows and step sizes
+// are staged in LDS with coalesced loads (the next chunk's loads are in
+// flight while this one is computed), softplus/exp run once per (token, head)
+// instead of once per lane, and y leaves through LDS as whole rows.
+constexpr int SCAN_TC = 16;  // tokens per chunk
+
+template <int R, int PC>
 __global__ void __launch_bounds__(256) ssd_scan_kernel(
     float* __restrict__ y, const float* __restrict__ xbc,
     const float* __restrict__ dt_raw_f32, const short* __restrict__ dt_raw_bf16,
@@ -105,11 +112,14 @@ __global__ void __launch_bounds__(256) ssd_scan_kernel(
     float* __restrict__ state, const long* __restrict__ positions,
     const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
     int heads, int groups, int P, int N) {
+  extern __shared__ float lds[];
+  constexpr int tc = SCAN_TC;
   const int s = blockIdx.z;
   const int h = blockIdx.y;
   const int ns = threadIdx.x & 15;
-  const int p = blockIdx.x * 16 + (threadIdx.x >> 4);
-  const bool p_ok = p < P;
+  const int pl = threadIdx.x >> 4;
+  const int p0 = blockIdx.x * (16 * PC);
+  const int pt = min(16 * PC, P - p0);  // columns of this tile
   const int first = cu_seqlens[s];
   const int len = cu_seqlens[s + 1] - first;
   if (len <= 0) return;
@@ -122,62 +132,119 @@ __global__ void __launch_bounds__(256) ssd_scan_kernel(
   const float bias = dt_bias[h];
   const float Dh = d_skip[h];
 
-  float S[R];
-  float* sp = state + ((slot * heads + h) * (long)P + (p_ok ? p : 0)) * N;
+  // LDS: B[tc][N] | C[tc][N] | x[tc][16 PC] | dt[tc] | decay[tc] | y[tc][16 PC]
+  const int XS = 16 * PC;
+  float* Bs = lds;
+  float* Cs = Bs + tc * N;
+  float* Xs = Cs + tc * N;
+  float* Ds = Xs + tc * XS;
+  float* As = Ds + tc;
+  float* Ys = As + tc;
+  float S[R][PC];
+  float* sp = state + ((slot * heads + h) * (long)P) * N;
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int n = ns + 16 * r;
-    S[r] = (!fresh && p_ok && n < N) ? sp[n] : 0.f;
-  }
-
-  auto load_dt = [&](int t) -> float {
-    const long i = (long)t * dt_stride + h;
-    return dt_raw_f32 ? dt_raw_f32[i] : bf16_bits_to_float(dt_raw_bf16[i]);
-  };
-
-  // operands of the token being processed, and of the next one (prefetch)
-  float Bn[R], Cn[R], xn, dtn;
-  auto fetch = [&](int t) {
-    const float* row = xbc + (long)t * channels;
-    xn = p_ok ? row[h * P + p] : 0.f;
-    dtn = load_dt(t);
+  for (int c = 0; c < PC; ++c) {
+    const int p = p0 + pl + 16 * c;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int n = ns + 16 * r;
-      const bool ok = n < N;
-      Bn[r] = ok ? row[inner + g * N + n] : 0.f;
-      Cn[r] = ok ? row[inner + groups * N + g * N + n] : 0.f;
+      S[r][c] = (!fresh && p < P && n < N) ? sp[(long)p * N + n] : 0.f;
+    }
+  }
+
+  // staging: 16 threads per token of the chunk, each takes every 16th
+  // element of the token's B, C and x rows (no index arithmetic beyond adds)
+  const int stk = threadIdx.x >> 4;   // token of the chunk this thread stages
+  const int sl = threadIdx.x & 15;
+  float sB[R], sC[R], sX[PC], sdt = 0.f;
+  auto prefetch = [&](int t0, int cnt) {
+    if (stk < cnt) {
+      const long t = first + t0 + stk;
+      const float* row = xbc + t * channels;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int n = sl + 16 * r;
+        sB[r] = n < N ? row[inner + g * N + n] : 0.f;
+        sC[r] = n < N ? row[inner + groups * N + g * N + n] : 0.f;
+      }
+#pragma unroll
+      for (int c = 0; c < PC; ++c) {
+        const int col = sl + 16 * c;
+        sX[c] = col < pt ? row[h * P + p0 + col] : 0.f;
+      }
+      if (sl == 0) {
+        const long i = t * dt_stride + h;
+        sdt = (dt_raw_f32 ? dt_raw_f32[i] : bf16_bits_to_float(dt_raw_bf16[i])) + bias;
+      }
     }
   };
-  fetch(first);
-  for (int i = 0; i < len; ++i) {
-    const int t = first + i;
-    float B[R], C[R];
+  auto commit = [&](int cnt) {
+    if (stk < cnt) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      B[r] = Bn[r];
-      C[r] = Cn[r];
-    }
-    const float x = xn;
-    const float v = dtn + bias;
-    if (i + 1 < len) fetch(t + 1);
-    // softplus without a clamp; log1p(exp(v)) overflows only past v ~ 88
-    const float dt = v > 30.f ? v : log1pf(expf(v));
-    const float a = expf(A * dt);
-    const float dtx = dt * x;
-    float acc = 0.f;
+      for (int r = 0; r < R; ++r) {
+        const int n = sl + 16 * r;
+        if (n < N) {
+          Bs[stk * N + n] = sB[r];
+          Cs[stk * N + n] = sC[r];
+        }
+      }
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      S[r] = a * S[r] + B[r] * dtx;
-      acc += S[r] * C[r];
+      for (int c = 0; c < PC; ++c) Xs[stk * XS + sl + 16 * c] = sX[c];
+      if (sl == 0) {
+        // softplus without a clamp; log1p(exp(v)) is v itself past v ~ 30
+        const float dt = sdt > 30.f ? sdt : log1pf(expf(sdt));
+        Ds[stk] = dt;
+        As[stk] = expf(A * dt);
+      }
     }
-    acc = group_reduce_sum<16>(acc);
-    if (ns == 0 && p_ok) y[(long)t * inner + h * P + p] = acc + Dh * x;
+  };
+
+  prefetch(0, min(tc, len));
+  for (int t0 = 0; t0 < len; t0 += tc) {
+    const int cnt = min(tc, len - t0);
+    __syncthreads();  // previous chunk's LDS fully consumed
+    commit(cnt);
+    __syncthreads();
+    if (t0 + tc < len) prefetch(t0 + tc, min(tc, len - t0 - tc));
+    for (int tk = 0; tk < cnt; ++tk) {
+      const float a = As[tk], dt = Ds[tk];
+      float B[R], C[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int n = ns + 16 * r;
+        const bool ok = n < N;
+        B[r] = ok ? Bs[tk * N + n] : 0.f;
+        C[r] = ok ? Cs[tk * N + n] : 0.f;
+      }
+#pragma unroll
+      for (int c = 0; c < PC; ++c) {
+        const int col = pl + 16 * c;
+        const float x = col < pt ? Xs[tk * XS + col] : 0.f;
+        const float dtx = dt * x;
+        float acc = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          S[r][c] = a * S[r][c] + B[r] * dtx;
+          acc += S[r][c] * C[r];
+        }
+        acc = group_reduce_sum<16>(acc);
+        if (ns == 0) Ys[tk * XS + col] = acc + Dh * x;
+      }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < cnt * pt; e += 256) {
+      const int tk = e / pt, col = e % pt;
+      y[(long)(first + t0 + tk) * inner + h * P + p0 + col] = Ys[tk * XS + col];
+    }
   }
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int n = ns + 16 * r;
-    if (p_ok && n < N) sp[n] = S[r];
+  for (int c = 0; c < PC; ++c) {
+    const int p = p0 + pl + 16 * c;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int n = ns + 16 * r;
+      if (p < P && n < N) sp[(long)p * N + n] = S[r][c];
+    }
   }
 }
 
@@ -223,15 +290,22 @@ extern "C" hipError_t ks_causal_conv_silu(
   return hipSuccess;
 }
 
-#define SSD_LAUNCH(RR)                                                        \
-  hipLaunchKernelGGL(ssd_scan_kernel<RR>, grid, dim3(256), 0, stream,         \
-                     (float*)y, (const float*)xbc,                            \
+#define SSD_LAUNCH(RR, PCC)                                                   \
+  hipLaunchKernelGGL((ssd_scan_kernel<RR, PCC>), grid, dim3(256), smem,       \
+                     stream, (float*)y, (const float*)xbc,                    \
                      dt_is_f32 ? (const float*)dt_raw : nullptr,              \
                      dt_is_f32 ? nullptr : (const short*)dt_raw, dt_stride,   \
                      (const float*)dt_bias, (const float*)a_log,              \
                      (const float*)d_skip, (float*)state,                     \
                      (const long*)positions, (const int*)cu_seqlens,          \
                      (const int*)slots, heads, groups, P, N)
+
+#define SSD_LAUNCH_R(RR)                                                      \
+  do {                                                                        \
+    if (pc == 1) SSD_LAUNCH(RR, 1);                                           \
+    else if (pc == 2) SSD_LAUNCH(RR, 2);                                      \
+    else SSD_LAUNCH(RR, 4);                                                   \
+  } while (0)
 
 extern "C" hipError_t ks_ssd_scan(void* y, const void* xbc, const void* dt_raw,
                                   long dt_stride, int dt_is_f32,
@@ -244,15 +318,21 @@ extern "C" hipError_t ks_ssd_scan(void* y, const void* xbc, const void* dt_raw,
   if (num_seqs == 0) return hipSuccess;
   if (groups <= 0 || heads % groups != 0 || N < 1 || N > 256)
     return hipErrorInvalidValue;
-  dim3 grid(cdiv(P, 16), heads, num_seqs);
+  // columns per lane: a block covers up to 64 columns of one head; wide
+  // state rows (R = 16) keep two columns so the state stays in registers
   const int R = cdiv(N, 16);
-  if (R <= 1) SSD_LAUNCH(1);
-  else if (R <= 2) SSD_LAUNCH(2);
-  else if (R <= 3) SSD_LAUNCH(3);
-  else if (R <= 4) SSD_LAUNCH(4);
-  else if (R <= 6) SSD_LAUNCH(6);
-  else if (R <= 8) SSD_LAUNCH(8);
-  else SSD_LAUNCH(16);
+  int pc = P > 32 ? 4 : (P > 16 ? 2 : 1);
+  if (R > 8 && pc > 2) pc = 2;
+  const int xs = 16 * pc;
+  const size_t smem = sizeof(float) * ((size_t)SCAN_TC * (2 * N + 2 * xs + 2));
+  dim3 grid(cdiv(P, xs), heads, num_seqs);
+  if (R <= 1) SSD_LAUNCH_R(1);
+  else if (R <= 2) SSD_LAUNCH_R(2);
+  else if (R <= 3) SSD_LAUNCH_R(3);
+  else if (R <= 4) SSD_LAUNCH_R(4);
+  else if (R <= 6) SSD_LAUNCH_R(6);
+  else if (R <= 8) SSD_LAUNCH_R(8);
+  else SSD_LAUNCH_R(16);
   HIP_CHECK_KERNEL();
   return hipSuccess;
 }

@@ -43,6 +43,13 @@ def detect_backend(model_dir: str) -> str:
     model_type = cfg.get("model_type", "")
     if model_type in ("llama", "mistral", "mixtral", "qwen2"):
         return "engine"
+    if "architecture" in cfg:
+        # designs outside the HF naming scheme that the engine's model
+        # registry knows (raises for unknown names)
+        from kserve_amd.models.registry import lookup
+
+        lookup(cfg["architecture"])
+        return "engine"
     if any(a.endswith(("ForCausalLM", "LMHeadModel")) for a in archs):
         # decoder the native engine doesn't implement: HF generate fallback
         # (reference generative_model.py behavior — request-serial)
@@ -70,12 +77,23 @@ def build_model(args):
             tp_size=getattr(args, "tensor_parallel_size", 1),
             pp_size=getattr(args, "pipeline_parallel_size", 1),
         )
-        from transformers import AutoTokenizer
+        from kserve_amd.models.registry import load_model_config
 
-        tokenizer = AutoTokenizer.from_pretrained(args.model_dir)
-        model_cfg = ModelConfig.from_hf_config(
-            os.path.join(args.model_dir, "config.json")
-        )
+        tokenizer = None
+        if any(
+            os.path.exists(os.path.join(args.model_dir, f))
+            for f in ("tokenizer.json", "tokenizer.model", "tokenizer_config.json")
+        ):
+            from transformers import AutoTokenizer
+
+            tokenizer = AutoTokenizer.from_pretrained(args.model_dir)
+        else:
+            logger.info("no tokenizer files: serving token-id prompts only")
+        # the registry picks the config (and later the model) class from
+        # config.json
+        model_cfg = load_model_config(args.model_dir)
+        if getattr(model_cfg, "dtype", None) and getattr(args, "dtype", None):
+            model_cfg.dtype = args.dtype
         if getattr(args, "expert_parallel", False):
             model_cfg.expert_parallel = True
         # draft-model speculation (vLLM --speculative-config equivalent)
@@ -149,6 +167,9 @@ def main(argv=None):
     parser.add_argument("--task", default=None)
     parser.add_argument("--tensor-parallel-size", dest="tensor_parallel_size", type=int, default=1)
     parser.add_argument("--pipeline-parallel-size", dest="pipeline_parallel_size", type=int, default=1)
+    parser.add_argument("--dtype", default=None, choices=["bfloat16", "float32"],
+                        help="activation/weight dtype of the engine (default: "
+                             "the model config's)")
     parser.add_argument("--max_model_len", type=int, default=8192)
     parser.add_argument("--max_num_seqs", type=int, default=256)
     # data-parallel contract flags (reference preset

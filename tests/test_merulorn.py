@@ -377,6 +377,12 @@ class TestConfigAndRegistry:
         assert mc.layers[2].mlp.limit == 2.5 and mc.layers[0].mlp is None
         assert native_modules_for(str(tmp_path)) == ("kserve_amd_seq_C",)
 
+    def test_server_cli_picks_the_engine(self, tmp_path):
+        from kserve_amd.runtimes.huggingfaceserver import detect_backend
+
+        (tmp_path / "config.json").write_text(json.dumps(two_kinds_config()))
+        assert detect_backend(str(tmp_path)) == "engine"
+
     def test_unknown_layer_type_is_refused(self):
         cfg = two_kinds_config()
         cfg["layers"][0]["type"] = "something-else"
