@@ -25,6 +25,33 @@ __global__ void clamped_swiglu_kernel(T* __restrict__ out,
   }
 }
 
+// 8 bf16 per lane when rows are 8-element aligned
+__global__ void clamped_swiglu_bf16x8_kernel(short* __restrict__ out,
+                                             const short* __restrict__ input,
+                                             const long rows, const int d,
+                                             const float alpha,
+                                             const float limit) {
+  const int nvec = d >> 3;
+  const short8_t* in_vec = reinterpret_cast<const short8_t*>(input);
+  short8_t* out_vec = reinterpret_cast<short8_t*>(out);
+  const long total = rows * nvec;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long row = idx / nvec;
+    const long col = idx % nvec;
+    const short8_t g8 = in_vec[row * (2 * nvec) + col];
+    const short8_t u8 = in_vec[row * (2 * nvec) + nvec + col];
+    short8_t o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float g = fminf(bf16_bits_to_float(g8[j]), limit);
+      const float u = fminf(fmaxf(bf16_bits_to_float(u8[j]), -limit), limit);
+      o[j] = float_to_bf16_bits(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+    }
+    out_vec[idx] = o;
+  }
+}
+
 __global__ void silu_and_mul_kernel(short* __restrict__ out,
                                     const short* __restrict__ input,
                                     const int rows, const int d) {
@@ -76,7 +103,15 @@ extern "C" hipError_t ks_clamped_swiglu(void* out, const void* input, int rows,
     hipLaunchKernelGGL(clamped_swiglu_kernel<float>, dim3(grid), dim3(256), 0,
                        stream, (float*)out, (const float*)input, (long)rows, d,
                        alpha, limit);
-  else
+  else if (d % 8 == 0 && ((uintptr_t)input % 16) == 0 &&
+           ((uintptr_t)out % 16) == 0) {
+    long tv = (long)rows * (d >> 3);
+    int gv = (int)((tv + 255) / 256);
+    if (gv > 8192) gv = 8192;
+    hipLaunchKernelGGL(clamped_swiglu_bf16x8_kernel, dim3(gv), dim3(256), 0,
+                       stream, (short*)out, (const short*)input, (long)rows, d,
+                       alpha, limit);
+  } else
     hipLaunchKernelGGL(clamped_swiglu_kernel<short>, dim3(grid), dim3(256), 0,
                        stream, (short*)out, (const short*)input, (long)rows, d,
                        alpha, limit);

@@ -83,65 +83,90 @@ __global__ void qk_norm_temp_cache_kernel(
   }
 }
 
-// 8 consecutive elements of a cache row -> fp32
+// 8 consecutive elements of a cache row, kept in the cache dtype while the
+// load is in flight (a bf16 chunk costs 4 registers) and widened on the way
+// into LDS
 template <typename T>
-__device__ __forceinline__ void load8(const T* p, bool vec, int valid, float* v);
+struct Chunk8;
 template <>
-__device__ __forceinline__ void load8<short>(const short* p, bool vec, int valid,
-                                             float* v) {
-  if (vec && valid >= 8) {
-    const short8_t x = *reinterpret_cast<const short8_t*>(p);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = bf16_bits_to_float(x[i]);
-  } else {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = i < valid ? bf16_bits_to_float(p[i]) : 0.f;
-  }
-}
-template <>
-__device__ __forceinline__ void load8<float>(const float* p, bool vec, int valid,
-                                             float* v) {
-  if (vec && valid >= 8) {
-    const f32x4 a = *reinterpret_cast<const f32x4*>(p);
-    const f32x4 b = *reinterpret_cast<const f32x4*>(p + 4);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v[i] = a[i];
-      v[4 + i] = b[i];
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = i < valid ? p[i] : 0.f;
-  }
-}
-
-// stage rows [k0, k0 + nk) of one kv head into LDS as fp32 [BK][WP + 4],
-// zero-filled past the head size and past nk
-template <typename T, int WP>
-__device__ __forceinline__ void stage_tile(float* dst, const T* cache,
-                                           const int* bt, int k0, int nk, int g,
-                                           int kv_heads, int W, int block_size,
-                                           bool vec) {
-  constexpr int CPR = WP / 8;  // 8-element chunks per row
-  constexpr int LS = WP + 4;
-  for (int c = threadIdx.x; c < BK * CPR; c += NT) {
-    const int j = c / CPR, d0 = (c % CPR) * 8;
-    float v[8];
-    const int valid = j < nk ? W - d0 : 0;
-    if (valid > 0) {
-      const int kp = k0 + j;
-      const long blk = bt[kp / block_size];
-      load8<T>(cache + ((blk * kv_heads + g) * block_size + kp % block_size) * W + d0,
-               vec, valid, v);
+struct Chunk8<short> {
+  short8_t x;
+  __device__ __forceinline__ void load(const short* p, bool vec, int valid) {
+    if (vec && valid >= 8) {
+      x = *reinterpret_cast<const short8_t*>(p);
     } else {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = 0.f;
+      for (int i = 0; i < 8; ++i) x[i] = i < valid ? p[i] : (short)0;
     }
-    f32x4* o = reinterpret_cast<f32x4*>(dst + j * LS + d0);
-    o[0] = f32x4{v[0], v[1], v[2], v[3]};
-    o[1] = f32x4{v[4], v[5], v[6], v[7]};
   }
-}
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = 0;
+  }
+  __device__ __forceinline__ float get(int i) const { return bf16_bits_to_float(x[i]); }
+};
+template <>
+struct Chunk8<float> {
+  f32x4 a, b;
+  __device__ __forceinline__ void load(const float* p, bool vec, int valid) {
+    if (vec && valid >= 8) {
+      a = *reinterpret_cast<const f32x4*>(p);
+      b = *reinterpret_cast<const f32x4*>(p + 4);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a[i] = i < valid ? p[i] : 0.f;
+        b[i] = 4 + i < valid ? p[4 + i] : 0.f;
+      }
+    }
+  }
+  __device__ __forceinline__ void zero() {
+    a = f32x4{0.f, 0.f, 0.f, 0.f};
+    b = a;
+  }
+  __device__ __forceinline__ float get(int i) const { return i < 4 ? a[i] : b[i - 4]; }
+};
+
+// rows [k0, k0 + nk) of one kv head, WP (padded width) columns: each thread
+// owns WP / 32 chunks of 8; fetch() issues the global loads, store() writes
+// them to LDS as fp32 [BK][WP + 4], zero past the head size and past nk
+template <typename T, int WP>
+struct TileStage {
+  static constexpr int CPR = WP / 8;          // chunks per row
+  static constexpr int NCH = BK * CPR / NT;   // chunks per thread
+  static constexpr int LS = WP + 4;
+  Chunk8<T> ch[NCH];
+
+  __device__ __forceinline__ void fetch(const T* cache, const int* bt, int k0,
+                                        int nk, int g, int kv_heads, int W,
+                                        int block_size, bool vec) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + NT * i;
+      const int j = c / CPR, d0 = (c % CPR) * 8;
+      const int valid = j < nk ? W - d0 : 0;
+      if (valid > 0) {
+        const int kp = k0 + j;
+        const long blk = bt[kp / block_size];
+        ch[i].load(
+            cache + ((blk * kv_heads + g) * block_size + kp % block_size) * W + d0,
+            vec, valid);
+      } else {
+        ch[i].zero();
+      }
+    }
+  }
+  __device__ __forceinline__ void store(float* dst) const {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + NT * i;
+      const int j = c / CPR, d0 = (c % CPR) * 8;
+      f32x4* o = reinterpret_cast<f32x4*>(dst + j * LS + d0);
+      o[0] = f32x4{ch[i].get(0), ch[i].get(1), ch[i].get(2), ch[i].get(3)};
+      o[1] = f32x4{ch[i].get(4), ch[i].get(5), ch[i].get(6), ch[i].get(7)};
+    }
+  }
+};
 
 template <typename T, int DP, int DVP, bool SPLITK>
 __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
@@ -204,12 +229,21 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   const bool kvec = (D % 8) == 0, vvec = (DV % 8) == 0;
   constexpr int KT = SPLITK ? 1 : 4;  // 16-key sub-tiles per wave and tile
 
+  // the next tile's global loads are in flight while this one is computed
+  TileStage<T, DP> kst;
+  TileStage<T, DVP> vst;
+  kst.fetch(k_cache, bt, 0, min(BK, last_pos + 1), g, kv_heads, D, block_size, kvec);
+  vst.fetch(v_cache, bt, 0, min(BK, last_pos + 1), g, kv_heads, DV, block_size, vvec);
   for (int k0 = 0; k0 <= last_pos; k0 += BK) {
     __syncthreads();  // previous tile fully consumed
-    const int nk = min(BK, last_pos + 1 - k0);
-    stage_tile<T, DP>(Ks, k_cache, bt, k0, nk, g, kv_heads, D, block_size, kvec);
-    stage_tile<T, DVP>(Vs, v_cache, bt, k0, nk, g, kv_heads, DV, block_size, vvec);
+    kst.store(Ks);
+    vst.store(Vs);
     __syncthreads();
+    if (k0 + BK <= last_pos) {
+      const int nn = min(BK, last_pos + 1 - (k0 + BK));
+      kst.fetch(k_cache, bt, k0 + BK, nn, g, kv_heads, D, block_size, kvec);
+      vst.fetch(v_cache, bt, k0 + BK, nn, g, kv_heads, DV, block_size, vvec);
+    }
     if (k0 > wave_last) continue;
 
     // S^T sub-tiles: acc[kt][v] = score(key k0 + 16 kt' + 4 lg + v, query li)

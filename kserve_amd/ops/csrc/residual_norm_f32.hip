@@ -61,6 +61,90 @@ __global__ void add_rms_norm_f32res_kernel(
   }
 }
 
+// 4 elements per lane and step, the row kept in registers between the two
+// passes (rows up to 256 * 4 * VEC_STEPS wide); picked by the launcher when
+// widths, strides and pointers are 4-element aligned
+constexpr int VEC_STEPS = 8;
+
+template <typename T>
+__device__ __forceinline__ void ld4(const T* p, float* v);
+template <>
+__device__ __forceinline__ void ld4<float>(const float* p, float* v) {
+  const float4_t x = *reinterpret_cast<const float4_t*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = x[i];
+}
+template <>
+__device__ __forceinline__ void ld4<short>(const short* p, float* v) {
+  const short4_t x = *reinterpret_cast<const short4_t*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = bf16_bits_to_float(x[i]);
+}
+template <typename T>
+__device__ __forceinline__ void st4(T* p, const float* v);
+template <>
+__device__ __forceinline__ void st4<float>(float* p, const float* v) {
+  *reinterpret_cast<float4_t*>(p) = float4_t{v[0], v[1], v[2], v[3]};
+}
+template <>
+__device__ __forceinline__ void st4<short>(short* p, const float* v) {
+  short4_t o;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = float_to_bf16_bits(v[i]);
+  *reinterpret_cast<short4_t*>(p) = o;
+}
+
+template <typename TD, typename TO>
+__global__ void add_rms_norm_f32res_vec4_kernel(
+    float* __restrict__ residual, const TD* __restrict__ d0, long d0_stride,
+    float s0, const TD* __restrict__ d1, long d1_stride, float s1,
+    const float* __restrict__ weight, float w_offset, float eps,
+    TO* __restrict__ out, int width) {
+  __shared__ float scratch[NW];
+  const long row = blockIdx.x;
+  float* r = residual + row * width;
+  float keep[VEC_STEPS][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < VEC_STEPS; ++k) {
+    const int i = (threadIdx.x + NT * k) * 4;
+    if (i < width) {
+      float v[4], d[4];
+      ld4<float>(r + i, v);
+      if (d0) {
+        ld4<TD>(d0 + row * d0_stride + i, d);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] += s0 * d[j];
+      }
+      if (d1) {
+        ld4<TD>(d1 + row * d1_stride + i, d);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] += s1 * d[j];
+      }
+      if (d0 || d1) st4<float>(r + i, v);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        keep[k][j] = v[j];
+        ss += v[j] * v[j];
+      }
+    }
+  }
+  ss = block_sum_sync<NW>(ss, scratch);
+  if (!out) return;
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+  for (int k = 0; k < VEC_STEPS; ++k) {
+    const int i = (threadIdx.x + NT * k) * 4;
+    if (i < width) {
+      float w[4], o[4];
+      ld4<float>(weight + i, w);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = keep[k][j] * inv * (w_offset + w[j]);
+      st4<TO>(out + row * width + i, o);
+    }
+  }
+}
+
 template <typename TZ, typename TO>
 __global__ void gated_group_rms_norm_kernel(TO* __restrict__ out,
                                             const float* __restrict__ y,
@@ -84,6 +168,46 @@ __global__ void gated_group_rms_norm_kernel(TO* __restrict__ out,
     const float zf = ld_f32(z, row * z_stride + g0 + i);
     const float v = y[row * inner + g0 + i] * (zf / (1.0f + expf(-zf)));
     st_f32(out, row * inner + g0 + i, v * inv * weight[g0 + i]);
+  }
+}
+
+template <typename TZ, typename TO>
+__global__ void gated_group_rms_norm_vec4_kernel(
+    TO* __restrict__ out, const float* __restrict__ y, const TZ* __restrict__ z,
+    long z_stride, const float* __restrict__ weight, float eps, int inner,
+    int group_size) {
+  __shared__ float scratch[NW];
+  const long row = blockIdx.x;
+  const int g0 = blockIdx.y * group_size;
+  float keep[VEC_STEPS][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < VEC_STEPS; ++k) {
+    const int i = (threadIdx.x + NT * k) * 4;
+    if (i < group_size) {
+      float yv[4], zv[4];
+      ld4<float>(y + row * inner + g0 + i, yv);
+      ld4<TZ>(z + row * z_stride + g0 + i, zv);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float v = yv[j] * (zv[j] / (1.0f + expf(-zv[j])));
+        keep[k][j] = v;
+        ss += v * v;
+      }
+    }
+  }
+  ss = block_sum_sync<NW>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)group_size + eps);
+#pragma unroll
+  for (int k = 0; k < VEC_STEPS; ++k) {
+    const int i = (threadIdx.x + NT * k) * 4;
+    if (i < group_size) {
+      float w[4], o[4];
+      ld4<float>(weight + g0 + i, w);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = keep[k][j] * inv * w[j];
+      st4<TO>(out + row * inner + g0 + i, o);
+    }
   }
 }
 
@@ -115,18 +239,30 @@ extern "C" hipError_t ks_add_rms_norm_f32res(
     long d1_stride, float s1, const void* weight, float w_offset, float eps,
     void* out, int rows, int width, int is_f32, hipStream_t stream) {
   if (rows == 0) return hipSuccess;
-  if (is_f32)
-    hipLaunchKernelGGL((add_rms_norm_f32res_kernel<float, float>), dim3(rows),
-                       dim3(NT), 0, stream, (float*)residual,
-                       (const float*)d0, d0_stride, s0, (const float*)d1,
-                       d1_stride, s1, (const float*)weight, w_offset, eps,
-                       (float*)out, width);
-  else
-    hipLaunchKernelGGL((add_rms_norm_f32res_kernel<short, short>), dim3(rows),
-                       dim3(NT), 0, stream, (float*)residual,
-                       (const short*)d0, d0_stride, s0, (const short*)d1,
-                       d1_stride, s1, (const float*)weight, w_offset, eps,
-                       (short*)out, width);
+  const int esz = is_f32 ? 4 : 2;
+  auto al = [](const void* p, int bytes) { return ((uintptr_t)p % bytes) == 0; };
+  const bool vec = width % 4 == 0 && width <= NT * 4 * VEC_STEPS &&
+                   d0_stride % 4 == 0 && d1_stride % 4 == 0 &&
+                   al(residual, 16) && al(weight, 16) && al(d0, 4 * esz) &&
+                   al(d1, 4 * esz) && al(out, 4 * esz);
+#define NORM_ARGS(TT)                                                         \
+  (float*)residual, (const TT*)d0, d0_stride, s0, (const TT*)d1, d1_stride,   \
+      s1, (const float*)weight, w_offset, eps, (TT*)out, width
+  if (is_f32) {
+    if (vec)
+      hipLaunchKernelGGL((add_rms_norm_f32res_vec4_kernel<float, float>),
+                         dim3(rows), dim3(NT), 0, stream, NORM_ARGS(float));
+    else
+      hipLaunchKernelGGL((add_rms_norm_f32res_kernel<float, float>), dim3(rows),
+                         dim3(NT), 0, stream, NORM_ARGS(float));
+  } else {
+    if (vec)
+      hipLaunchKernelGGL((add_rms_norm_f32res_vec4_kernel<short, short>),
+                         dim3(rows), dim3(NT), 0, stream, NORM_ARGS(short));
+    else
+      hipLaunchKernelGGL((add_rms_norm_f32res_kernel<short, short>), dim3(rows),
+                         dim3(NT), 0, stream, NORM_ARGS(short));
+  }
   HIP_CHECK_KERNEL();
   return hipSuccess;
 }
@@ -140,16 +276,33 @@ extern "C" hipError_t ks_gated_group_rms_norm(void* out, const void* y,
   if (rows == 0) return hipSuccess;
   if (groups <= 0 || inner % groups != 0) return hipErrorInvalidValue;
   const int gs = inner / groups;
-  if (is_f32)
-    hipLaunchKernelGGL((gated_group_rms_norm_kernel<float, float>),
-                       dim3(rows, groups), dim3(NT), 0, stream, (float*)out,
-                       (const float*)y, (const float*)z, z_stride,
-                       (const float*)weight, eps, inner, gs);
-  else
-    hipLaunchKernelGGL((gated_group_rms_norm_kernel<short, short>),
-                       dim3(rows, groups), dim3(NT), 0, stream, (short*)out,
-                       (const float*)y, (const short*)z, z_stride,
-                       (const float*)weight, eps, inner, gs);
+  const int esz = is_f32 ? 4 : 2;
+  const bool vec = gs % 4 == 0 && gs <= NT * 4 * VEC_STEPS && z_stride % 4 == 0 &&
+                   ((uintptr_t)y % 16) == 0 && ((uintptr_t)weight % 16) == 0 &&
+                   ((uintptr_t)z % (4 * esz)) == 0 &&
+                   ((uintptr_t)out % (4 * esz)) == 0;
+#define GNORM_ARGS(TT)                                                        \
+  (TT*)out, (const float*)y, (const TT*)z, z_stride, (const float*)weight,    \
+      eps, inner, gs
+  if (is_f32) {
+    if (vec)
+      hipLaunchKernelGGL((gated_group_rms_norm_vec4_kernel<float, float>),
+                         dim3(rows, groups), dim3(NT), 0, stream,
+                         GNORM_ARGS(float));
+    else
+      hipLaunchKernelGGL((gated_group_rms_norm_kernel<float, float>),
+                         dim3(rows, groups), dim3(NT), 0, stream,
+                         GNORM_ARGS(float));
+  } else {
+    if (vec)
+      hipLaunchKernelGGL((gated_group_rms_norm_vec4_kernel<short, short>),
+                         dim3(rows, groups), dim3(NT), 0, stream,
+                         GNORM_ARGS(short));
+    else
+      hipLaunchKernelGGL((gated_group_rms_norm_kernel<short, short>),
+                         dim3(rows, groups), dim3(NT), 0, stream,
+                         GNORM_ARGS(short));
+  }
   HIP_CHECK_KERNEL();
   return hipSuccess;
 }

@@ -63,6 +63,68 @@ __global__ void causal_conv_silu_kernel(
   out[(long)t * channels + c] = silu_f(acc);
 }
 
+// 4 consecutive channels per lane (8- or 16-byte loads, 16-byte stores); the
+// launcher picks it when pointers, strides and the channel count allow
+template <typename T>
+__device__ __forceinline__ void load4(const T* p, float* v);
+template <>
+__device__ __forceinline__ void load4<short>(const short* p, float* v) {
+  const short4_t x = *reinterpret_cast<const short4_t*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = bf16_bits_to_float(x[i]);
+}
+template <>
+__device__ __forceinline__ void load4<float>(const float* p, float* v) {
+  const float4_t x = *reinterpret_cast<const float4_t*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = x[i];
+}
+
+constexpr int CONV_TT = 8;  // tokens per block of the vector kernel
+
+template <typename T, int TAPS>
+__global__ void causal_conv_silu_vec4_kernel(
+    float* __restrict__ out, const T* __restrict__ in, long in_stride,
+    const float* __restrict__ w, const float* __restrict__ bias,
+    const T* __restrict__ conv_state, const long* __restrict__ positions,
+    const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ slots, int tokens, int channels) {
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (c >= channels) return;
+  constexpr int hist = TAPS - 1;
+  // taps and bias of this lane's 4 channels, reused for every token
+  float wt[4][TAPS], b4[4];
+  load4<float>(bias + c, b4);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) wt[i][j] = w[(long)(c + i) * TAPS + j];
+  const int t_end = min(tokens, (int)(blockIdx.y + 1) * CONV_TT);
+  for (int t = blockIdx.y * CONV_TT; t < t_end; ++t) {
+    const int s = seq_of_token[t];
+    const int first = cu_seqlens[s];
+    const long pos = positions[t];
+    const long slot = slots[s];
+    float acc[4] = {b4[0], b4[1], b4[2], b4[3]};
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) {
+      const int back = hist - j;
+      if (pos - back < 0) continue;
+      float v[4];
+      if (t - back >= first)
+        load4<T>(in + (long)(t - back) * in_stride + c, v);
+      else
+        load4<T>(conv_state + (slot * hist + (hist - back + (t - first))) * channels + c, v);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] += wt[i][j] * v[i];
+    }
+    float4_t o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = silu_f(acc[i]);
+    *reinterpret_cast<float4_t*>(out + (long)t * channels + c) = o;
+  }
+}
+
 template <typename T>
 __global__ void conv_state_update_kernel(
     T* __restrict__ conv_state, const T* __restrict__ in, long in_stride,
@@ -104,7 +166,8 @@ __global__ void conv_state_update_kernel(
 constexpr int SCAN_TC = 16;  // tokens per chunk
 
 template <int R, int PC>
-__global__ void __launch_bounds__(256) ssd_scan_kernel(
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4)))
+ssd_scan_kernel(
     float* __restrict__ y, const float* __restrict__ xbc,
     const float* __restrict__ dt_raw_f32, const short* __restrict__ dt_raw_bf16,
     long dt_stride, const float* __restrict__ dt_bias,
@@ -259,13 +322,32 @@ extern "C" hipError_t ks_causal_conv_silu(
   if (taps < 1 || taps > MAX_TAPS) return hipErrorInvalidValue;
   dim3 grid(cdiv(channels, 256), tokens);
   dim3 grid_u(cdiv(channels, 256), num_seqs);
+  const int esz = is_f32 ? 4 : 2;
+  // 4-channel vectors need every row start on a 4-element boundary
+  const bool vec = channels % 4 == 0 && in_stride % 4 == 0 &&
+                   ((uintptr_t)in % (4 * esz)) == 0 &&
+                   ((uintptr_t)conv_state % (4 * esz)) == 0 &&
+                   ((uintptr_t)out % 16) == 0 && ((uintptr_t)bias % 16) == 0 &&
+                   taps >= 2 && taps <= 4;
+  dim3 grid_v(cdiv(channels / 4, 256), cdiv(tokens, CONV_TT));
+#define CONV_ARGS(TT)                                                         \
+  (float*)out, (const TT*)in, in_stride, (const float*)w, (const float*)bias, \
+      (const TT*)conv_state, (const long*)positions,                          \
+      (const int*)seq_of_token, (const int*)cu_seqlens, (const int*)slots
+#define CONV_VEC_K(TT, K)                                                     \
+  hipLaunchKernelGGL((causal_conv_silu_vec4_kernel<TT, K>), grid_v,           \
+                     dim3(256), 0, stream, CONV_ARGS(TT), tokens, channels)
+#define CONV_VEC(TT)                                                          \
+  do {                                                                        \
+    if (taps == 2) CONV_VEC_K(TT, 2);                                         \
+    else if (taps == 3) CONV_VEC_K(TT, 3);                                    \
+    else CONV_VEC_K(TT, 4);                                                   \
+  } while (0)
   if (is_f32) {
-    hipLaunchKernelGGL(causal_conv_silu_kernel<float>, grid, dim3(256), 0,
-                       stream, (float*)out, (const float*)in, in_stride,
-                       (const float*)w, (const float*)bias,
-                       (const float*)conv_state, (const long*)positions,
-                       (const int*)seq_of_token, (const int*)cu_seqlens,
-                       (const int*)slots, channels, taps);
+    if (vec) CONV_VEC(float);
+    else
+      hipLaunchKernelGGL(causal_conv_silu_kernel<float>, grid, dim3(256), 0,
+                         stream, CONV_ARGS(float), channels, taps);
     if (taps > 1)
       hipLaunchKernelGGL(conv_state_update_kernel<float>, grid_u, dim3(256), 0,
                          stream, (float*)conv_state, (const float*)in,
@@ -273,12 +355,10 @@ extern "C" hipError_t ks_causal_conv_silu(
                          (const int*)cu_seqlens, (const int*)slots, channels,
                          taps);
   } else {
-    hipLaunchKernelGGL(causal_conv_silu_kernel<short>, grid, dim3(256), 0,
-                       stream, (float*)out, (const short*)in, in_stride,
-                       (const float*)w, (const float*)bias,
-                       (const short*)conv_state, (const long*)positions,
-                       (const int*)seq_of_token, (const int*)cu_seqlens,
-                       (const int*)slots, channels, taps);
+    if (vec) CONV_VEC(short);
+    else
+      hipLaunchKernelGGL(causal_conv_silu_kernel<short>, grid, dim3(256), 0,
+                         stream, CONV_ARGS(short), channels, taps);
     if (taps > 1)
       hipLaunchKernelGGL(conv_state_update_kernel<short>, grid_u, dim3(256), 0,
                          stream, (short*)conv_state, (const short*)in,
