@@ -11,7 +11,7 @@ PropagateModelStatus requeues every second until ready
 (components/predictor.go:285-289); Stopped-condition teardown
 (controller.go:306-338).
 
-The desired manifests come from reconciler.desired_state (the round-1 pure
+The desired manifests come from reconciler.desired_state (the pure
 renderer); this module is the loop around it: apply with owner references
 and semantic diff, prune orphans, set status conditions, requeue until the
 Deployments report available.

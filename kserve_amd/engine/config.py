@@ -51,7 +51,7 @@ class ModelConfig:
     rope_scaling: Optional[dict] = None
     # Mistral-style sliding-window size from the HF config; enforced in
     # all three attention kernels (decode/flash/paged-context) as an
-    # absolute-position bound since round 2.
+    # absolute-position bound.
     sliding_window: int = None
 
     def __post_init__(self):

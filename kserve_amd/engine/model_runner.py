@@ -659,7 +659,7 @@ class ModelRunner:
         the fused temperature/top-k/top-p Gumbel sampler runs IN-GRAPH, the
         seed buffer advances in-replay, and greedy rows are overridden by
         argmax — so multi-step windows work for temperature>0 batches
-        (round-1 limitation: windows were greedy-only)."""
+        (not only for greedy ones)."""
         g = self._sampled_graphs.get(bs)
         if g is not None:
             return g

@@ -69,7 +69,7 @@ class NoNativeExtension(RuntimeError):
     """Raised when a GPU tensor reaches an op whose HIP extension is missing.
 
     The MI355X compute path must never fall back to eager torch silently on
-    a GPU box (the round-end harness records which .so files were loaded).
+    a GPU box (a silent fallback would hide a missing build).
     """
 
     def __init__(self, op: str, detail: str = ""):

@@ -1,6 +1,6 @@
 """Custom op dispatch: CDNA4 HIP kernels on GPU, torch reference on CPU.
 
-Policy (round-end harness contract): GPU tensors MUST run the native
+Policy: GPU tensors MUST run the native
 extension — if ``kserve_amd_C`` is missing on a CUDA/ROCm device the op
 raises ``NoNativeExtension`` instead of silently falling back to eager
 torch. CPU tensors use the fp32 torch reference (tests, engine logic).

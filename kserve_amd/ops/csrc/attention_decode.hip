@@ -166,7 +166,7 @@ __global__ __launch_bounds__(256, OCC) void paged_attention_kernel(
         v_cache + (((long)block_id * num_kv_heads + kv_head) * PAGE) * D;
 
     if constexpr (MQ && HPW == 1 && V4) {
-      // ---- MFMA QK (round-2 experiment): the page's 16 tokens form the
+      // ---- MFMA QK (experiment): the page's 16 tokens form the
       // B columns of four 16x16x32 MFMA steps (K^T fragments are
       // contiguous 16-B reads: lane reads dims (lane>>4)*8 of token
       // lane&15), freeing the VALU dot + 4-lane reduce entirely. Scores

@@ -172,7 +172,7 @@ void paged_attention_decode(at::Tensor& out, at::Tensor& q,
   // gains (S=64: 3.75->3.96 at 4 splits) and tiny batches need deep
   // splits (S=8: 0.71 unsplit vs 1.6-1.7 at 8-16). Rule: group<=4 AND
   // base<=512 -> clamp(2048/base, 2, 8); otherwise split only below
-  // 512 workgroups (the round-1 rule).
+  // 512 workgroups (the original rule).
   int n_splits = 1;
   long base_wgs = (long)S * Hkv;
   const int grp = H / Hkv;
@@ -385,6 +385,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   def_sampling(m);
   m.def("skinny_gemm", &skinny_gemm, "decode GEMM (N<=256, MFMA streaming)");
   m.def("gemm8", &gemm8,
-        "EXPERIMENTAL 8-phase 256x256 MFMA GEMM (round-2 candidate)");
+        "EXPERIMENTAL 8-phase 256x256 MFMA GEMM");
   m.def("mfma_probe", &mfma_probe, "MFMA layout probe (tests)");
 }

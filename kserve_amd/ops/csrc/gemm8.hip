@@ -1,4 +1,4 @@
-// 8-phase 256x256 MFMA GEMM (EXPERIMENTAL — round-2 candidate).
+// 8-phase 256x256 MFMA GEMM (EXPERIMENTAL).
 //
 // Plain-HIP port of the verified 8-phase schedule from the CDNA4 guide
 // ("The 256-sq 8-phase template", measured 1563 TF @4k / 1728 @8k on
@@ -7,9 +7,9 @@
 // C-quadrant (4Mx2N fragments) x K=64 per phase, counted vmcnt at phases
 // 4/8 only, s_setprio(1) around the MFMA burst.
 //
-// Status: UNVALIDATED ON HARDWARE in round 1 (written after the GPU
+// Status: first written without hardware validation (written after the GPU
 // budget was spent). Gated off everywhere: the dispatcher never selects
-// it unless KS_GEMM8=1, and its GPU test requires KS_GEMM8=1. Round 2:
+// it unless KS_GEMM8=1, and its GPU test requires KS_GEMM8=1. Later:
 // run tests/test_gpu_ops.py -k gemm8 + tools/gemm8_bench.py first thing.
 //
 // Computes D[M,N] = A[M,K] @ W[N,K]^T (torch F.linear convention), bf16
@@ -360,7 +360,7 @@ __global__ __launch_bounds__(512, 1) void gemm8_kernel(
 }
 
 // Half-granular 8-phase schedule (guide T3+T4, the full counted-vmcnt
-// discipline; NEXT.md round-3 item 1). One 16 KiB stage unit per phase,
+// discipline; counted-vmcnt pipeline). One 16 KiB stage unit per phase,
 // issued in future-consumption order, landing checked by ONE counted
 // s_waitcnt vmcnt(4) per K-tile (never 0 in the main loop):
 //

@@ -295,7 +295,7 @@ def test_logit_bias(engine):
 
 
 class TestSampledWindows:
-    """Multi-step decode windows at temperature>0 (round-2: the in-graph
+    """Multi-step decode windows at temperature>0 (the in-graph
     fused sampler removes the greedy-only window restriction; CPU exercises
     the eager path of ModelRunner.multi_step_decode(sampled=True))."""
 

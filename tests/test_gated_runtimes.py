@@ -1,7 +1,7 @@
 """Import-gated runtime predict paths exercised against stub libraries.
 
 xgboost/lightgbm/paddle/pypmml are absent from this offline image, so
-round 1 never ran these runtimes' predict logic. These tests inject
+earlier versions never ran these runtimes' predict logic. These tests inject
 minimal stand-ins implementing exactly the API surface each runtime
 calls (the reference's mock-based storage tests play the same role), so
 the V1/V2 plumbing, file discovery, and error mapping are verified even

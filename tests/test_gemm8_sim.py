@@ -5,7 +5,7 @@ permutation (global_load_lds chunks + optional st_16x32 swizzle), the
 per-phase LDS fragment reads, and the MFMA 16x16x32 fragment contract
 (layouts verified on hardware by mfma_probe). If this reproduces
 A @ W^T bit-for-math, the kernel's indexing is correct and only
-synchronization remains to validate on the GPU in round 2.
+synchronization remains to validate on the GPU.
 """
 
 import numpy as np

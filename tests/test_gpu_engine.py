@@ -383,7 +383,7 @@ def test_prefix_cache_on_gpu():
 
 def test_mixtral_moe_on_gpu():
     """MoE engine path on GPU: decode is hipGraph-captured via the
-    dense-bmm path (round 2); batched greedy equals single greedy."""
+    dense-bmm path; batched greedy equals single greedy."""
     from kserve_amd.engine.config import (
         CacheConfig,
         EngineConfig,
@@ -431,7 +431,7 @@ def test_mixtral_moe_on_gpu():
 
 
 def test_sampled_window_graph_topk1_matches_greedy():
-    """In-graph sampled decode (round 2): with top_k=1 the fused sampler
+    """In-graph sampled decode: with top_k=1 the fused sampler
     must reproduce greedy tokens exactly, through the SAMPLED graph variant
     (multi-step windows at temperature>0)."""
     from kserve_amd.engine.engine import LLMEngine

@@ -473,7 +473,7 @@ class TestSkinnyGemm:
 
 class TestGemm8Experimental:
     """8-phase MFMA GEMM (experimental; not in the serving path).
-    GPU-validated round 2 across the full SW x SCHED matrix — runs by
+    GPU-validated across the full SW x SCHED matrix — runs by
     default now; KS_GEMM8=0 skips."""
 
     @pytest.mark.skipif(

@@ -133,7 +133,7 @@ def test_guided_choice_shared_prefix():
 
 
 class TestSchemaMachine:
-    """json_schema structured outputs (round 2): byte-level acceptance of
+    """json_schema structured outputs: byte-level acceptance of
     the strict compact serialization, rejection of shape violations."""
 
     def _m(self, schema):

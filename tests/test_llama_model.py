@@ -426,7 +426,7 @@ class TestLlama31RopeScaling:
 class TestSlidingWindow:
     """Sliding-window attention (Mistral-family): beyond the window the
     outputs must match an explicitly-masked full-attention reference, and
-    must DIFFER from unwindowed attention (round-1 recorded the window but
+    must DIFFER from unwindowed attention (an earlier version recorded the window but
     attended the full context)."""
 
     def _refs(self, T=24, W=8, H=2, D=16):
@@ -529,7 +529,7 @@ class TestSlidingWindow:
 
 
 class TestMoEDensePath:
-    """Capture-safe dense-bmm MoE decode (round 2): the dense path must be
+    """Capture-safe dense-bmm MoE decode: the dense path must be
     numerically identical to the token-bucketed sparse loop (routing enters
     only through the zero-masked mix)."""
 

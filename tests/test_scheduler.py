@@ -196,7 +196,7 @@ def test_decode_not_starved_when_seats_full():
 
 
 def test_window_capped_not_disabled_when_admission_blocked():
-    """Round 2: a waiting request that cannot be admitted (seats full) no
+    """A waiting request that cannot be admitted (seats full) no
     longer forces one-token decode steps — the window is capped to
     BLOCKED_ADMISSION_WINDOW instead (it was unschedulable this step
     either way)."""

@@ -152,7 +152,7 @@ def test_all_features_combined_matches_plain():
 
 
 class TestDraftModelSpeculation:
-    """Draft-MODEL speculation (round 2): exact greedy outputs regardless
+    """Draft-MODEL speculation: exact greedy outputs regardless
     of draft quality; a perfect draft (same weights) accepts everything."""
 
     def _engine(self, draft_seed_offset=1, k=3):
