@@ -23,9 +23,27 @@
 //    tiles x heads x sequences, so decode batches fill the chip).
 #include "dtype_io.h"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int MAX_TAPS = 16;
+
+// sum over each row of 16 lanes with DPP lane swaps (VALU rate, no LDS
+// traffic): swap within pairs, within quads, mirror the 8-lane half, mirror
+// the row; every lane of the row ends with the row's sum
+__device__ __forceinline__ float row16_sum(float v) {
+  auto swz = [](float x, auto ctrl) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x),
+                                           decltype(ctrl)::value, 0xF, 0xF, true));
+  };
+  v += swz(v, std::integral_constant<int, 0xB1>{});   // quad_perm [1,0,3,2]
+  v += swz(v, std::integral_constant<int, 0x4E>{});   // quad_perm [2,3,0,1]
+  v += swz(v, std::integral_constant<int, 0x141>{});  // row_half_mirror
+  v += swz(v, std::integral_constant<int, 0x140>{});  // row_mirror
+  return v;
+}
 
 __device__ __forceinline__ float silu_f(float v) {
   return v / (1.0f + expf(-v));
@@ -290,7 +308,7 @@ ssd_scan_kernel(
           S[r][c] = a * S[r][c] + B[r] * dtx;
           acc += S[r][c] * C[r];
         }
-        acc = group_reduce_sum<16>(acc);
+        acc = row16_sum(acc);
         if (ns == 0) Ys[tk * XS + col] = acc + Dh * x;
       }
     }
