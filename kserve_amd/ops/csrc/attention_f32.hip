@@ -17,7 +17,8 @@
 //    and the S^T accumulator registers are already the B operand of
 //    O^T += V^T P^T (the contraction runs over keys in the accumulator's own
 //    order; V is read from LDS in that order), so the weights never leave
-//    registers.
+//    registers. The head-dimension contraction and the value columns are
+//    likewise assigned to lanes so that every LDS operand read is 16 bytes.
 //    Prefill: a block takes 64 consecutive tokens of one query head, 16 per
 //    wave, all waves sharing the staged K/V tile. Decode (one token per
 //    sequence): a block takes the query heads of one KV group as its 16
@@ -139,7 +140,7 @@ struct TileStage {
 
   __device__ __forceinline__ void fetch(const T* cache, const int* bt, int k0,
                                         int nk, int g, int kv_heads, int W,
-                                        int block_size, bool vec) {
+                                        int block_size, int bs_shift, bool vec) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int c = threadIdx.x + NT * i;
@@ -147,10 +148,12 @@ struct TileStage {
       const int valid = j < nk ? W - d0 : 0;
       if (valid > 0) {
         const int kp = k0 + j;
-        const long blk = bt[kp / block_size];
-        ch[i].load(
-            cache + ((blk * kv_heads + g) * block_size + kp % block_size) * W + d0,
-            vec, valid);
+        // bs_shift >= 0: pages of 2^bs_shift tokens (no integer division)
+        const int pb = bs_shift >= 0 ? kp >> bs_shift : kp / block_size;
+        const int po = bs_shift >= 0 ? kp & (block_size - 1) : kp % block_size;
+        const long blk = bt[pb];
+        ch[i].load(cache + ((blk * kv_heads + g) * block_size + po) * W + d0, vec,
+                   valid);
       } else {
         ch[i].zero();
       }
@@ -212,13 +215,17 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   const int wave_last =
       SPLITK ? last_pos : base_pos + min(wave * 16 + 15, nrows - 1) / hpb;
 
-  // Q^T fragments (B operand): lane (k = lg, column li) of k-step ks holds
-  // q[query li][4 ks + lg], pre-multiplied by the softmax scale
+  // Q^T fragments (B operand). The contraction over the head dimension may
+  // run in any order as long as both operands agree: k-step ks of lane group
+  // lg stands for d = lg * DP/4 + ks, so a lane's K values are contiguous in
+  // LDS (16-byte reads) and so are its q values here. Pre-multiplied by the
+  // softmax scale and log2(e): the softmax runs on exp2.
+  const float qscale = scale * 1.44269504088896340736f;
   float qf[DP / 4];
 #pragma unroll
   for (int ks = 0; ks < DP / 4; ++ks) {
-    const int d = 4 * ks + lg;
-    qf[ks] = (row_ok && d < D) ? q[((long)tok * heads + hd) * D + d] * scale : 0.f;
+    const int d = lg * (DP / 4) + ks;
+    qf[ks] = (row_ok && d < D) ? q[((long)tok * heads + hd) * D + d] * qscale : 0.f;
   }
   f32x4 o[DVP / 16];
 #pragma unroll
@@ -227,13 +234,15 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
 
   const int* bt = block_tables + (long)s * bt_stride;
   const bool kvec = (D % 8) == 0, vvec = (DV % 8) == 0;
+  const int bs_shift =
+      (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1;
   constexpr int KT = SPLITK ? 1 : 4;  // 16-key sub-tiles per wave and tile
 
   // the next tile's global loads are in flight while this one is computed
   TileStage<T, DP> kst;
   TileStage<T, DVP> vst;
-  kst.fetch(k_cache, bt, 0, min(BK, last_pos + 1), g, kv_heads, D, block_size, kvec);
-  vst.fetch(v_cache, bt, 0, min(BK, last_pos + 1), g, kv_heads, DV, block_size, vvec);
+  kst.fetch(k_cache, bt, 0, min(BK, last_pos + 1), g, kv_heads, D, block_size, bs_shift, kvec);
+  vst.fetch(v_cache, bt, 0, min(BK, last_pos + 1), g, kv_heads, DV, block_size, bs_shift, vvec);
   for (int k0 = 0; k0 <= last_pos; k0 += BK) {
     __syncthreads();  // previous tile fully consumed
     kst.store(Ks);
@@ -241,23 +250,35 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     __syncthreads();
     if (k0 + BK <= last_pos) {
       const int nn = min(BK, last_pos + 1 - (k0 + BK));
-      kst.fetch(k_cache, bt, k0 + BK, nn, g, kv_heads, D, block_size, kvec);
-      vst.fetch(v_cache, bt, k0 + BK, nn, g, kv_heads, DV, block_size, vvec);
+      kst.fetch(k_cache, bt, k0 + BK, nn, g, kv_heads, D, block_size, bs_shift, kvec);
+      vst.fetch(v_cache, bt, k0 + BK, nn, g, kv_heads, DV, block_size, bs_shift, vvec);
     }
     if (k0 > wave_last) continue;
 
     // S^T sub-tiles: acc[kt][v] = score(key k0 + 16 kt' + 4 lg + v, query li)
-    f32x4 sc[KT];
+    // k-steps outermost, two accumulators per sub-tile: 2 KT independent
+    // MFMA chains are in flight instead of one long dependent one
+    f32x4 sc[KT], sc2[KT];
 #pragma unroll
     for (int t = 0; t < KT; ++t) {
-      const int kt = SPLITK ? wave : t;
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-      const float* ka = Ks + (16 * kt + li) * KS + lg;
-#pragma unroll
-      for (int ks = 0; ks < DP / 4; ++ks)
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[4 * ks], qf[ks], acc, 0, 0, 0);
-      sc[t] = acc;
+      sc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      sc2[t] = sc[t];
     }
+#pragma unroll
+    for (int k4 = 0; k4 < DP / 16; ++k4) {
+#pragma unroll
+      for (int t = 0; t < KT; ++t) {
+        const int kt = SPLITK ? wave : t;
+        const f32x4 kv = *reinterpret_cast<const f32x4*>(
+            Ks + (16 * kt + li) * KS + lg * (DP / 4) + 4 * k4);
+        sc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[0], qf[4 * k4 + 0], sc[t], 0, 0, 0);
+        sc2[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[1], qf[4 * k4 + 1], sc2[t], 0, 0, 0);
+        sc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[2], qf[4 * k4 + 2], sc[t], 0, 0, 0);
+        sc2[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[3], qf[4 * k4 + 3], sc2[t], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < KT; ++t) sc[t] += sc2[t];
     float mt = -INFINITY;
 #pragma unroll
     for (int t = 0; t < KT; ++t) {
@@ -273,13 +294,13 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     mt = fmaxf(mt, __shfl_xor(mt, 32, WAVE_SIZE));
     const float mn = fmaxf(m, mt);
     // a column that has seen no visible key yet keeps mn = -inf
-    const float corr = (mn == -INFINITY) ? 1.f : expf(m - mn);
+    const float corr = (mn == -INFINITY) ? 1.f : exp2f(m - mn);
     float ps = 0.f;
 #pragma unroll
     for (int t = 0; t < KT; ++t)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const float pv = sc[t][v] == -INFINITY ? 0.f : expf(sc[t][v] - mn);
+        const float pv = sc[t][v] == -INFINITY ? 0.f : exp2f(sc[t][v] - mn);
         sc[t][v] = pv;
         ps += pv;
       }
@@ -295,11 +316,18 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
       const int kt = SPLITK ? wave : t;
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const float* va = Vs + (16 * kt + 4 * lg + v) * VS + li;
+        // row li of output tile i is value column 64 (i/4) + 4 li + i%4: the
+        // four tiles of a 64-column block come from one 16-byte read
+        const f32x4* va = reinterpret_cast<const f32x4*>(
+            Vs + (16 * kt + 4 * lg + v) * VS + 4 * li);
         const float pb = sc[t][v];
 #pragma unroll
-        for (int i = 0; i < DVP / 16; ++i)
-          o[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(va[16 * i], pb, o[i], 0, 0, 0);
+        for (int j = 0; j < DVP / 64; ++j) {
+          const f32x4 vv = va[16 * j];
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+            o[4 * j + c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[c], pb, o[4 * j + c], 0, 0, 0);
+        }
       }
     }
   }
@@ -318,7 +346,7 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     for (int i = 0; i < DVP / 16; ++i)
 #pragma unroll
       for (int v = 0; v < 4; ++v)
-        Os[(wave * 16 + li) * DVP + 16 * i + 4 * lg + v] = o[i][v];
+        Os[(wave * 16 + li) * DVP + 64 * (i / 4) + 4 * (4 * lg + v) + i % 4] = o[i][v];
     __syncthreads();
     for (int e = threadIdx.x; e < nrows * DVP; e += NT) {
       const int row = e / DVP, dv = e % DVP;
@@ -330,7 +358,7 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
 #pragma unroll
       for (int w = 0; w < NW; ++w) {
         const float mw = Ms[w * 16 + row];
-        const float f = mw == -INFINITY ? 0.f : expf(mw - M);
+        const float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
         L += Ls[w * 16 + row] * f;
         O += Os[(w * 16 + row) * DVP + dv] * f;
       }
@@ -355,7 +383,7 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   for (int i = 0; i < DVP / 16; ++i)
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      const int dv = 16 * i + 4 * lg + v;
+      const int dv = 64 * (i / 4) + 4 * (4 * lg + v) + i % 4;
       if (dv < DV) st_f32(out, ((long)tok * heads + hd) * DV + dv, o[i][v] * f);
     }
 }
