@@ -392,6 +392,10 @@ class SchedulerConfig:
     max_model_len: int = 8192
     # chunked prefill: cap on prompt tokens scheduled per step
     enable_chunked_prefill: bool = False
+    # mixed batches: a step that prefills also carries one decode token of
+    # every running request (through the paged-context path), so running
+    # requests keep producing while prompts are admitted
+    mixed_batches: bool = False
     # multi-step decode: consecutive greedy decode iterations run as pure
     # hipGraph replays (sampled token fed back on-GPU); stop conditions are
     # applied after the window. 1 disables.

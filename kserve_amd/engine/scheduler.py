@@ -203,9 +203,33 @@ class Scheduler:
             batch.requests.append(req)
             batch.num_scheduled_tokens.append(n_new)
             token_budget -= n_new
+        decoders = list(self.running)
         for r in batch.requests:
             self.running.append(r)
+        if batch.requests and self.config.mixed_batches:
+            self._add_decode_tokens(batch, decoders, token_budget)
         return batch
+
+    def _add_decode_tokens(
+        self, batch: ScheduledBatch, decoders: List[Request], token_budget: int
+    ) -> None:
+        """Mixed batch: give every already-running request its next decode
+        token in this prefill step, as far as the token budget and the free
+        pages (above the watermark) allow. A request that does not fit simply
+        waits for the next step; nothing is preempted for a rider."""
+        bm = self.block_manager
+        for req in decoders:
+            if token_budget <= 0:
+                break
+            if req.num_computed_tokens != req.num_tokens - 1:
+                continue  # mid-prefill or not ready for a decode token
+            need = bm.blocks_needed(req.num_tokens) - len(bm.get_block_table(req))
+            if need > 0 and bm.num_free_blocks - need < bm.watermark_blocks:
+                continue
+            bm.append_slot(req)
+            batch.requests.append(req)
+            batch.num_scheduled_tokens.append(1)
+            token_budget -= 1
 
     def _schedule_decode(self) -> ScheduledBatch:
         batch = ScheduledBatch(is_prefill=False)

@@ -118,6 +118,7 @@ def build_model(args):
             scheduler=SchedulerConfig(
                 max_num_seqs=getattr(args, "max_num_seqs", 256),
                 max_model_len=getattr(args, "max_model_len", 8192),
+                mixed_batches=getattr(args, "mixed_batches", False),
                 speculative_ngram=getattr(args, "speculative_ngram", 0),
                 speculative_k=(
                     getattr(args, "num_speculative_tokens", 3)
@@ -170,6 +171,10 @@ def main(argv=None):
     parser.add_argument("--dtype", default=None, choices=["bfloat16", "float32"],
                         help="activation/weight dtype of the engine (default: "
                              "the model config's)")
+    parser.add_argument("--enable-mixed-batches", dest="mixed_batches",
+                        action="store_true",
+                        help="prefill steps also carry one decode token of "
+                             "every running request")
     parser.add_argument("--max_model_len", type=int, default=8192)
     parser.add_argument("--max_num_seqs", type=int, default=256)
     # data-parallel contract flags (reference preset

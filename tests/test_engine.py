@@ -370,3 +370,38 @@ class TestSampledWindows:
         # no windows: one token per step (prefill samples the first token,
         # then 5 single-token decode steps)
         assert steps >= 6
+
+
+def test_mixed_batches_same_tokens_as_separate_steps():
+    """mixed_batches (decode tokens riding with prefill steps) changes the
+    batching, not the greedy result — llama path, paged-context attention."""
+    def run(mixed):
+        torch.manual_seed(0)
+        cfg = EngineConfig(
+            model=ModelConfig.tiny(vocab_size=128),
+            cache=CacheConfig(block_size=4, num_gpu_blocks=128),
+            scheduler=SchedulerConfig(
+                max_num_seqs=8, max_num_batched_tokens=12, max_model_len=128,
+                multi_step=1, mixed_batches=mixed,
+            ),
+            device="cpu", eos_token_id=-1,
+        )
+        eng = LLMEngine(cfg)
+        mixed_steps = 0
+        inner = eng.runner.execute_prefill
+
+        def spy(batch, bm, logit_rows=None):
+            nonlocal mixed_steps
+            ns = batch.num_scheduled_tokens
+            mixed_steps += int(min(ns) == 1 and max(ns) > 1)
+            return inner(batch, bm, logit_rows=logit_rows)
+
+        eng.runner.execute_prefill = spy
+        prompts = [list(range(1, 11)), list(range(20, 29)), list(range(40, 51))]
+        out = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=6))
+        return [o.output_token_ids for o in out.values()], mixed_steps
+
+    plain, n0 = run(False)
+    mixed, n1 = run(True)
+    assert n0 == 0 and n1 > 0
+    assert plain == mixed

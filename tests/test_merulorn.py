@@ -55,7 +55,8 @@ def two_kinds_config(**kw):
 
 
 def make_engine(cfg, sd, backend, num_blocks=64, block_size=16, max_seqs=4,
-                eager=False, multi_step=1, max_len=512):
+                eager=False, multi_step=1, max_len=512, batched_tokens=None,
+                mixed=False):
     device, dtype = backend
     mc = HybridModelConfig.from_dict(cfg)
     mc.dtype = dtype
@@ -65,9 +66,10 @@ def make_engine(cfg, sd, backend, num_blocks=64, block_size=16, max_seqs=4,
         model=mc,
         cache=CacheConfig(block_size=block_size, num_gpu_blocks=num_blocks),
         scheduler=SchedulerConfig(
-            max_num_seqs=max_seqs, max_num_batched_tokens=max_len,
+            max_num_seqs=max_seqs,
+            max_num_batched_tokens=batched_tokens or max_len,
             max_model_len=max_len, enable_chunked_prefill=True,
-            multi_step=multi_step,
+            multi_step=multi_step, mixed_batches=mixed,
         ),
         device=device, eos_token_id=-1, enforce_eager=eager,
     )
@@ -370,6 +372,30 @@ class TestGeneration:
                 if (top2[0] - top2[1]).item() > 1e-3:
                     assert int(logits.argmax()) == t
                 seq.append(t)
+
+    def test_mixed_batches_in_the_scheduler(self, backend):
+        """With a token budget that admits one prompt per step, running
+        requests ride along with the next prompt's prefill; the tokens are
+        the same as without riders."""
+        cfg = two_kinds_config()
+        sd = weights_for(cfg, backend, seed=18)
+        prompts = [random_prompt(n, cfg["vocab"], 90 + n) for n in (20, 18, 21)]
+        sp = SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True)
+        plain = make_engine(cfg, sd, backend, batched_tokens=24).generate(prompts, sp)
+        eng = make_engine(cfg, sd, backend, batched_tokens=24, mixed=True)
+        seen = []
+        inner = eng.runner.execute_prefill
+
+        def spy(batch, bm, logit_rows=None):
+            seen.append(sorted(batch.num_scheduled_tokens))
+            return inner(batch, bm, logit_rows=logit_rows)
+
+        eng.runner.execute_prefill = spy
+        mixed = eng.generate(prompts, sp)
+        assert any(b[0] == 1 and b[-1] > 1 for b in seen), seen
+        if backend[1] == "float32":
+            for a, b in zip(plain.values(), mixed.values()):
+                assert a.output_token_ids == b.output_token_ids
 
     def test_chunked_admission_and_preemption(self, backend):
         """A pool that cannot hold all requests: the scheduler preempts, the

@@ -230,3 +230,32 @@ def test_window_capped_not_disabled_when_admission_blocked():
     assert not batch.is_prefill
     k = eng.scheduler.reserve_decode_window(batch, 8)
     assert k == eng.scheduler.BLOCKED_ADMISSION_WINDOW  # capped, not 1
+
+
+def test_mixed_batches_carry_decode_tokens():
+    """mixed_batches: a prefill step also schedules one token of each
+    running request that is ready to decode, within the token budget."""
+    from kserve_amd.engine.config import CacheConfig, SchedulerConfig
+    from kserve_amd.engine.request import Request
+    from kserve_amd.engine.sampling_params import SamplingParams
+    from kserve_amd.engine.scheduler import Scheduler
+
+    s = Scheduler(
+        SchedulerConfig(max_num_seqs=8, max_num_batched_tokens=12,
+                        max_model_len=64, mixed_batches=True),
+        CacheConfig(block_size=4), 64,
+    )
+    a = Request("a", list(range(10)), SamplingParams(max_tokens=8))
+    b = Request("b", list(range(9)), SamplingParams(max_tokens=8))
+    s.add_request(a)
+    s.add_request(b)
+    first = s.schedule()
+    assert [r.request_id for r in first.requests] == ["a"]  # b does not fit
+    a.num_computed_tokens = 10
+    a.append_output_token(3)
+    second = s.schedule()
+    assert second.is_prefill
+    assert [(r.request_id, n) for r, n in
+            zip(second.requests, second.num_scheduled_tokens)] == [("b", 9), ("a", 1)]
+    assert s.running.count(a) == 1
+    assert len(s.block_manager.get_block_table(a)) * 4 >= 11
