@@ -180,10 +180,19 @@ class AttentionMixerSpec:
     scale: float
     q_temp_coef: float = 0.0
     q_temp_every: int = 0
+    # rotary positions on the first ``rot_dims`` coordinates of every q/k
+    # head (coordinate i pairs with i + rot_dims/2); 0 = no rotation
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    # chunk-local causal mask: a query sees only keys of its own block of
+    # ``chunk`` positions (counted from position 0); 0 = plain causal
+    chunk: int = 0
 
     @classmethod
     def from_dict(cls, d: dict) -> "AttentionMixerSpec":
         qt = d.get("q_temp") or {}
+        rot = d.get("rot") or {}
+        mask = d.get("mask") or {}
         return cls(
             heads=int(d["heads"]),
             kv_heads=int(d.get("kv_heads", d["heads"])),
@@ -192,6 +201,9 @@ class AttentionMixerSpec:
             scale=float(d["scale"]),
             q_temp_coef=float(qt.get("coef", 0.0)),
             q_temp_every=int(qt.get("every", 0)),
+            rot_dims=int(rot.get("dims", 0)),
+            rot_base=float(rot.get("base", 10000.0)),
+            chunk=int(mask.get("size", 0)),
         )
 
 
@@ -250,6 +262,49 @@ class GLUSpec:
 
 
 @dataclass
+class MoESpec:
+    """Mixture of clamped gated experts: each token runs the ``top`` experts
+    with the largest sigmoid router scores; the (un-normalised) score scales
+    the expert's INPUT. An optional shared expert runs for every token."""
+
+    experts: int
+    top: int
+    ff: int
+    limit: float
+    shared: Optional[GLUSpec] = None
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "MoESpec":
+        sh = d.get("shared")
+        return cls(
+            experts=int(d["router"]["experts"]),
+            top=int(d["router"]["top"]),
+            ff=int(d["expert"]["ff"]),
+            limit=float(d["expert"]["limit"]),
+            shared=GLUSpec(ff=int(sh["ff"]), limit=float(sh["limit"])) if sh else None,
+        )
+
+
+def feed_forward_spec(d: Optional[dict]):
+    """``mlp`` entry of a layer -> GLUSpec, MoESpec or None."""
+    if not d:
+        return None
+    if d.get("kind", "moe" if "router" in d else "dense") == "moe":
+        return MoESpec.from_dict(d)
+    return GLUSpec.from_dict(d)
+
+
+@dataclass
+class LoopSpec:
+    """Layers ``start .. stop-1`` run ``times`` times in a row with the same
+    weights (every pass with a cache of its own) before the rest follow."""
+
+    start: int = 0
+    stop: int = 0
+    times: int = 1
+
+
+@dataclass
 class HybridLayerSpec:
     """One pre-norm layer: a mixer made of an attention branch and/or a
     state-space branch reading the same normed input (outputs summed with
@@ -260,7 +315,7 @@ class HybridLayerSpec:
     ssm: Optional[SSMMixerSpec] = None
     attention_scale: float = 1.0
     ssm_scale: float = 1.0
-    mlp: Optional[GLUSpec] = None
+    mlp: Optional[object] = None  # GLUSpec or MoESpec
 
 
 @dataclass
@@ -279,10 +334,24 @@ class HybridModelConfig:
     # fields the engine reads on every model config
     num_local_experts: int = 0
     sliding_window: Optional[int] = None
+    loop: Optional[LoopSpec] = None
 
     @property
     def num_layers(self) -> int:
         return len(self.layers)
+
+    def layer_runs(self) -> list:
+        """Execution order as (layer index, pass number or None): a looped
+        span appears once per pass. Every run has a cache of its own."""
+        n = len(self.layers)
+        lp = self.loop
+        if lp is None or lp.stop <= lp.start:
+            return [(i, None) for i in range(n)]
+        runs = [(i, None) for i in range(lp.start)]
+        for t in range(lp.times):
+            runs += [(i, t) for i in range(lp.start, lp.stop)]
+        runs += [(i, None) for i in range(lp.stop, n)]
+        return runs
 
     @property
     def has_recurrent_state(self) -> bool:
@@ -290,9 +359,10 @@ class HybridModelConfig:
 
     def kv_bytes_per_block(self, block_size: int, itemsize: int) -> int:
         return sum(
-            l.attention.kv_heads * (l.attention.dim + l.attention.vdim)
-            for l in self.layers
-            if l.attention is not None
+            self.layers[i].attention.kv_heads
+            * (self.layers[i].attention.dim + self.layers[i].attention.vdim)
+            for i, _ in self.layer_runs()
+            if self.layers[i].attention is not None
         ) * block_size * itemsize
 
     @classmethod
@@ -301,8 +371,14 @@ class HybridModelConfig:
         for entry in cfg["layers"]:
             kind = entry["type"]
             mixer = entry["mixer"]
-            mlp = GLUSpec.from_dict(entry["mlp"]) if entry.get("mlp") else None
-            if kind == "mamba2":
+            mlp = feed_forward_spec(entry.get("mlp"))
+            if kind == "attention":
+                layers.append(
+                    HybridLayerSpec(
+                        kind, attention=AttentionMixerSpec.from_dict(mixer), mlp=mlp
+                    )
+                )
+            elif kind == "mamba2":
                 layers.append(
                     HybridLayerSpec(kind, ssm=SSMMixerSpec.from_dict(mixer), mlp=mlp)
                 )
@@ -327,6 +403,15 @@ class HybridModelConfig:
             embedding_scale=float(cfg.get("embedding", {}).get("scale", 1.0)),
             model_name=model_name,
             architecture=cfg.get("architecture", "Merulorn"),
+            loop=(
+                LoopSpec(
+                    start=int(cfg["loop"].get("start", 0)),
+                    stop=int(cfg["loop"].get("stop", 0)),
+                    times=int(cfg["loop"].get("times", 1)),
+                )
+                if cfg.get("loop")
+                else None
+            ),
         )
 
     @classmethod

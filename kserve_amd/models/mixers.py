@@ -21,7 +21,13 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from kserve_amd import ops
-from kserve_amd.engine.config import AttentionMixerSpec, GLUSpec, SSMMixerSpec
+from kserve_amd.engine.config import (
+    AttentionMixerSpec,
+    GLUSpec,
+    MoESpec,
+    SSMMixerSpec,
+)
+from kserve_amd.ops.torch_ref import rotary_inv_freq
 
 
 class LayerCache(NamedTuple):
@@ -155,6 +161,79 @@ class NormedGatedAttention(nn.Module):
         )
 
 
+class RotaryChunkSinkAttention(nn.Module):
+    """Softmax attention with per-head q/k RMS norm (weights of size ``dim``
+    shared by the heads), rotary positions on the first ``rot_dims``
+    coordinates, fp32 scores against the paged cache, and three optional
+    parts: a chunk-local causal mask (``spec.chunk``), a learned per-head
+    sink term in the softmax denominator (``sink``), and unit-norm values
+    that are rotated by their own position over all of ``vdim`` before they
+    are cached, with every head output turned back by the query's position
+    (``value_unit_norm`` / ``rotate_values``). No biases, no gate. The
+    q|k|v projections are one fused GEMM."""
+
+    def __init__(
+        self, width: int, spec: AttentionMixerSpec, eps: float, dtype,
+        sink: bool = True, value_unit_norm: bool = True,
+        rotate_values: bool = True,
+    ):
+        super().__init__()
+        self.spec = spec
+        self.eps = eps
+        self.dtype = dtype
+        self.q_w = spec.heads * spec.dim
+        self.k_w = spec.kv_heads * spec.dim
+        self.v_w = spec.kv_heads * spec.vdim
+        if spec.rot_dims % 2 or spec.rot_dims > spec.dim:
+            raise ValueError("rot dims must be even and at most the head size")
+        if rotate_values and spec.vdim % 2:
+            raise ValueError("rotated values need an even value size")
+        self.qkv = _param(self.q_w + self.k_w + self.v_w, width, dtype=dtype)
+        self.q_norm = _param(spec.dim, dtype=torch.float32)
+        self.k_norm = _param(spec.dim, dtype=torch.float32)
+        self.sink = _param(spec.heads, dtype=torch.float32) if sink else None
+        self.o_proj = _param(width, spec.heads * spec.vdim, dtype=dtype)
+        self.value_unit_norm = value_unit_norm
+        self.register_buffer(
+            "qk_inv_freq",
+            rotary_inv_freq(spec.rot_dims, spec.rot_base) if spec.rot_dims else None,
+            persistent=False,
+        )
+        self.register_buffer(
+            "v_inv_freq",
+            rotary_inv_freq(spec.vdim, spec.rot_base) if rotate_values else None,
+            persistent=False,
+        )
+
+    def load(self, get, prefix: str):
+        dt = self.dtype
+        self.qkv.copy_(
+            torch.cat([get(prefix + n).to(dt) for n in ("q", "k", "v")], dim=0)
+        )
+        self.q_norm.copy_(get(prefix + "q.norm").float())
+        self.k_norm.copy_(get(prefix + "k.norm").float())
+        if self.sink is not None:
+            self.sink.copy_(get(prefix + "sink").float())
+        self.o_proj.copy_(get(prefix + "o").to(dt))
+
+    def forward(self, h, positions, cache: LayerCache, meta):
+        s = self.spec
+        proj = F.linear(h, self.qkv)
+        a, b = self.q_w, self.q_w + self.k_w
+        qn = ops.qk_headnorm_rope_cache(
+            proj[:, :a], proj[:, a:b], proj[:, b:], self.q_norm, self.k_norm,
+            positions, meta.slot_mapping, cache.k, cache.v, self.eps, s.heads,
+            self.qk_inv_freq, self.value_unit_norm, self.v_inv_freq,
+        )
+        o = ops.ctx_attention_f32(
+            qn, cache.k, cache.v, meta.block_tables, meta.cu_seqlens,
+            meta.context_lens, s.scale, meta.max_seqlen, s.heads,
+            out_dtype=self.dtype, sink=self.sink, chunk=s.chunk,
+            out_inv_freq=self.v_inv_freq,
+        )
+        return F.linear(o, self.o_proj)
+
+
 class ClampedGLU(nn.Module):
     """y = g * sigmoid(alpha g) * (u + 1), g = min(W_gate h, limit),
     u = clamp(W_up h, -limit, limit); gate|up are one fused GEMM."""
@@ -179,3 +258,120 @@ class ClampedGLU(nn.Module):
             F.linear(h, self.gate_up), self.ALPHA, self.spec.limit
         )
         return F.linear(act, self.down)
+
+
+class RoutedClampedMoE(nn.Module):
+    """Mixture of clamped gated experts. Router logits are fp32; a token runs
+    the ``top`` experts with the largest scores (sigmoid, used as they are),
+    each on the token's input TIMES its score, and the expert outputs are
+    summed in fp32 together with an optional always-on shared expert.
+
+    Expert weights are stacked ([E, 2 ff, width] gate|up and [E, width, ff]).
+    Small batches and captured decode graphs run every expert on every token
+    (a GEMM pair per expert) with zero input rows for the experts a token did
+    not choose (an expert without biases maps zero to zero, so nothing has to
+    be masked afterwards): static shapes, no host synchronisation. Larger
+    batches sort the (token, expert) pairs by expert and run one GEMM pair
+    per expert on its contiguous rows."""
+
+    ALPHA = ClampedGLU.ALPHA
+    # the all-experts form does experts/top times the arithmetic of the sorted
+    # one; it is used while that factor times the batch stays below this many
+    # token-rows (where reading the expert weights dominates anyway)
+    DENSE_ROW_BUDGET = 1024
+
+    def __init__(self, width: int, spec: MoESpec, dtype):
+        super().__init__()
+        self.spec = spec
+        self.dtype = dtype
+        E = spec.experts
+        # batches up to this size take the all-experts form, eager or
+        # captured; decode graphs are captured up to it and larger decode
+        # batches run eager steps through the sorted form
+        self.dense_max_tokens = max(16, self.DENSE_ROW_BUDGET * spec.top // E)
+        if not 1 <= spec.top <= E:
+            raise ValueError("top must be between 1 and the number of experts")
+        self.router = _param(E, width, dtype=torch.float32)
+        self.gate_up = _param(E, 2 * spec.ff, width, dtype=dtype)
+        self.down = _param(E, width, spec.ff, dtype=dtype)
+        self.shared = (
+            ClampedGLU(width, spec.shared, dtype) if spec.shared is not None else None
+        )
+
+    def load(self, get, prefix: str):
+        dt = self.dtype
+        self.router.copy_(get(prefix + "router").float())
+        for e in range(self.spec.experts):
+            p = f"{prefix}e{e}."
+            self.gate_up[e].copy_(
+                torch.cat([get(p + "gate").to(dt), get(p + "up").to(dt)], dim=0)
+            )
+            self.down[e].copy_(get(p + "down").to(dt))
+        if self.shared is not None:
+            self.shared.load(get, prefix + "shared.")
+
+    def _dense(self, h, dense_w, extra):
+        E, T = self.spec.experts, h.shape[0]
+        ar = torch.arange(T, dtype=torch.int32, device=h.device)
+        # row e*T + t = h[t] * weight[t, e] (zero where e was not chosen)
+        xb = ops.gather_scale_rows(
+            h, ar.repeat(E), dense_w.t().contiguous().view(-1)
+        ).view(E, T, -1)
+        # one plain GEMM per expert: the same library call every dense layer
+        # makes, and as safe inside a captured graph
+        gu = torch.empty((E, T, 2 * self.spec.ff), dtype=h.dtype, device=h.device)
+        for e in range(E):
+            torch.mm(xb[e], self.gate_up[e].t(), out=gu[e])
+        act = ops.clamped_swiglu(
+            gu.view(E * T, -1), self.ALPHA, self.spec.limit
+        ).view(E, T, -1)
+        ye = torch.empty((E, T, h.shape[1]), dtype=h.dtype, device=h.device)
+        for e in range(E):
+            torch.mm(act[e], self.down[e].t(), out=ye[e])
+        ye = ye.view(E * T, -1)
+        # token t's E rows are e*T + t
+        index = (
+            ar.view(T, 1) + T * torch.arange(E, dtype=torch.int32, device=h.device)
+        ).view(-1)
+        return ops.combine_rows(ye, index, E, extra)
+
+    def _sorted(self, h, idx, w, extra):
+        E, top = self.spec.experts, self.spec.top
+        flat = idx.view(-1).long()
+        order = torch.sort(flat, stable=True).indices
+        counts = torch.bincount(flat, minlength=E).tolist()  # host sync
+        xs = ops.gather_scale_rows(
+            h, (order // top).to(torch.int32), w.view(-1)[order]
+        )
+        n = xs.shape[0]
+        gu = torch.empty((n, 2 * self.spec.ff), dtype=h.dtype, device=h.device)
+        a = 0
+        for e, c in enumerate(counts):
+            if c:
+                torch.mm(xs[a : a + c], self.gate_up[e].t(), out=gu[a : a + c])
+            a += c
+        act = ops.clamped_swiglu(gu, self.ALPHA, self.spec.limit)
+        ys = torch.empty((n, h.shape[1]), dtype=h.dtype, device=h.device)
+        a = 0
+        for e, c in enumerate(counts):
+            if c:
+                torch.mm(act[a : a + c], self.down[e].t(), out=ys[a : a + c])
+            a += c
+        # pair p = t*top + k sits at sorted row inv[p]
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(n, device=h.device)
+        return ops.combine_rows(ys, inv.to(torch.int32), top, extra)
+
+    def forward(self, h):
+        """[T, width] in the activation dtype -> fp32 [T, width]."""
+        T = h.shape[0]
+        extra = self.shared(h) if self.shared is not None else None
+        dense = T <= self.dense_max_tokens or (
+            h.is_cuda and torch.cuda.is_current_stream_capturing()
+        )
+        idx, w, dense_w, _ = ops.route_tokens(
+            h, self.router, self.spec.top, dense=dense
+        )
+        if dense:
+            return self._dense(h, dense_w, extra)
+        return self._sorted(h, idx, w, extra)

@@ -44,6 +44,12 @@ register(
     "kserve_amd.models.merulorn.MerulornForCausalLM",
     ("kserve_amd_seq_C",),
 )
+register(
+    "Desalix",
+    "kserve_amd.engine.config.HybridModelConfig",
+    "kserve_amd.models.desalix.DesalixForCausalLM",
+    ("kserve_amd_seq_C",),
+)
 
 
 def architecture_of(config_json: dict) -> str:

@@ -336,6 +336,7 @@ def embed_scale_sinpos(table, tokens, positions, inv_freq, scale: float):
     position * inv_freq (the start of an fp32 residual stream)."""
     if table.is_cuda:
         out = _f32_like(tokens.shape[0], table.shape[1], table)
+        # inv_freq None: no positional term
         _native_seq("embed_scale_sinpos").embed_scale_sinpos(
             out, table, tokens, positions, inv_freq, float(scale)
         )
@@ -427,7 +428,13 @@ def qk_norm_temp_cache(
 def ctx_attention_f32(
     q, k_cache, v_cache, block_tables, cu_q, ctx_lens, scale: float,
     max_q_len: int, heads: int, gate=None, out_dtype=torch.float32,
+    sink=None, chunk: int = 0, out_inv_freq=None,
 ):
+    """Paged causal attention with fp32 scores and weights. Optional parts:
+    ``gate`` [T, heads] (output times sigmoid), ``sink`` [heads] fp32 (one
+    more term exp(sink) in the softmax denominator), ``chunk`` (a query sees
+    only keys of its own block of that many positions), ``out_inv_freq``
+    [vdim/2] fp32 (each head output turned back by its query position)."""
     if q.is_cuda:
         out = torch.empty(
             (q.shape[0], heads * v_cache.shape[3]), dtype=out_dtype,
@@ -435,13 +442,119 @@ def ctx_attention_f32(
         )
         _native_seq("ctx_attention_f32").ctx_attention_f32(
             out, q, k_cache, v_cache, block_tables, cu_q, ctx_lens, gate,
-            float(scale), int(max_q_len), int(heads),
+            float(scale), int(max_q_len), int(heads), sink, int(chunk),
+            out_inv_freq,
         )
         return out
     return torch_ref.ctx_attention_f32(
         q, k_cache, v_cache, block_tables, cu_q, ctx_lens, scale, heads,
-        gate, out_dtype,
+        gate, out_dtype, sink, chunk, out_inv_freq,
     )
+
+
+def qk_headnorm_rope_cache(
+    q, k, v, qw, kw, positions, slot_mapping, k_cache, v_cache, eps: float,
+    heads: int, qk_inv_freq=None, v_unit_norm: bool = False, v_inv_freq=None,
+):
+    """Per-head q/k RMS norm (weights [dim]) + rotary positions, optional
+    unit-norm and rotation of the values, KV page scatter; returns q fp32."""
+    if q.is_cuda:
+        q_out = _f32_like(q.shape[0], q.shape[1], q)
+        _native_seq("qk_headnorm_rope_cache").qk_headnorm_rope_cache(
+            q_out, q, k, v, qw, kw, positions, slot_mapping, k_cache, v_cache,
+            float(eps), int(heads), qk_inv_freq, bool(v_unit_norm), v_inv_freq,
+        )
+        return q_out
+    return torch_ref.qk_headnorm_rope_cache(
+        q, k, v, qw, kw, positions, slot_mapping, k_cache, v_cache, eps,
+        heads, qk_inv_freq, v_unit_norm, v_inv_freq,
+    )
+
+
+def post_norm_add_rms_norm(
+    residual, delta, post_gain: float, layer_scale, eps: float,
+    next_gain: float, out_dtype, add_rows=None, add_vec=None,
+    want_out: bool = True,
+):
+    """Close one sandwich-normed sublayer and open the next in one pass over
+    the fp32 residual (in place): += layer_scale * scalar-gain RMS norm of the
+    sublayer output, += optional per-token rows and one shared row, then the
+    scalar-gain RMS norm of the result in ``out_dtype``."""
+    if residual.is_cuda:
+        out = (
+            torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+            if want_out else None
+        )
+        _native_seq("post_norm_add_rms_norm").post_norm_add_rms_norm(
+            residual, delta, float(post_gain), layer_scale, float(eps),
+            float(next_gain), out, add_rows, add_vec,
+        )
+        return out
+    return torch_ref.post_norm_add_rms_norm(
+        residual, delta, post_gain, layer_scale, eps, next_gain, out_dtype,
+        add_rows, add_vec, want_out,
+    )
+
+
+def router_topk(
+    logits, top: int, softmax: bool = False, renorm: bool = False,
+    dense: bool = False,
+):
+    """fp32 router logits [T, E] -> (expert ids int32 [T, top], weights fp32
+    [T, top], dense [T, E] weights or None) by sigmoid (or softmax) score."""
+    if logits.is_cuda:
+        T, E = logits.shape
+        idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+        w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+        dw = (
+            torch.empty((T, E), dtype=torch.float32, device=logits.device)
+            if dense else None
+        )
+        _native_seq("router_topk").router_topk(
+            idx, w, dw, logits, bool(softmax), bool(renorm)
+        )
+        return idx, w, dw
+    return torch_ref.router_topk(logits, top, softmax, renorm, dense)
+
+
+def route_tokens(
+    h, router, top: int, softmax: bool = False, renorm: bool = False,
+    dense: bool = False, want_logits: bool = False,
+):
+    """The router in one kernel: fp32 logits of h [T, W] (activation dtype)
+    against fp32 router rows [E, W], scores, the ``top`` experts. Returns
+    (expert ids int32 [T, top], weights fp32 [T, top], dense [T, E] weights or
+    None, logits fp32 [T, E] or None)."""
+    if h.is_cuda:
+        T, E = h.shape[0], router.shape[0]
+        dev = h.device
+        idx = torch.empty((T, top), dtype=torch.int32, device=dev)
+        w = torch.empty((T, top), dtype=torch.float32, device=dev)
+        dw = torch.empty((T, E), dtype=torch.float32, device=dev) if dense else None
+        lg = torch.empty((T, E), dtype=torch.float32, device=dev) if want_logits else None
+        _native_seq("route_tokens").route_tokens(
+            idx, w, dw, lg, h, router, bool(softmax), bool(renorm)
+        )
+        return idx, w, dw, lg
+    return torch_ref.route_tokens(h, router, top, softmax, renorm, dense, want_logits)
+
+
+def gather_scale_rows(x, rows, scales):
+    """out[r] = x[rows[r]] * scales[r] in x's dtype (rows int32, scales fp32)."""
+    if x.is_cuda:
+        out = torch.empty((rows.numel(), x.shape[1]), dtype=x.dtype, device=x.device)
+        _native_seq("gather_scale_rows").gather_scale_rows(out, x, rows, scales)
+        return out
+    return torch_ref.gather_scale_rows(x, rows, scales)
+
+
+def combine_rows(y, index, top: int, extra=None):
+    """fp32 out[t] = sum_k y[index[t*top + k]] (+ extra[t])."""
+    if y.is_cuda:
+        out = _f32_like(index.numel() // top, y.shape[1], y)
+        _native_seq("combine_rows").combine_rows(out, y, index, int(top), extra)
+        return out
+    return torch_ref.combine_rows(y, index, top, extra)
 
 
 def clamped_swiglu(x, alpha: float, limit: float):

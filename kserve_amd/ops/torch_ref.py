@@ -326,6 +326,8 @@ def sinusoid_inv_freq(width: int, base: float = 10000.0) -> torch.Tensor:
 
 
 def embed_scale_sinpos(table, tokens, positions, inv_freq, scale: float):
+    if inv_freq is None:
+        return table[tokens].float() * scale
     width = table.shape[1]
     ang = positions.to(torch.float32).unsqueeze(1) * inv_freq.unsqueeze(0)
     pe = torch.stack([torch.sin(ang), torch.cos(ang)], dim=-1).reshape(
@@ -435,7 +437,8 @@ def qk_norm_temp_cache(
 
 def ctx_attention_f32(
     q, k_cache, v_cache, block_tables, cu_q, ctx_lens, scale: float,
-    heads: int, gate=None, out_dtype=torch.float32,
+    heads: int, gate=None, out_dtype=torch.float32, sink=None, chunk: int = 0,
+    out_inv_freq=None,
 ):
     _, G, bs, D = k_cache.shape
     DV = v_cache.shape[3]
@@ -456,12 +459,148 @@ def ctx_attention_f32(
         qs = q[a:b].reshape(b - a, heads, D).float().transpose(0, 1)
         sc = torch.matmul(qs, K.transpose(1, 2)) * scale  # [heads, n, ctx]
         qpos = torch.arange(ctx - (b - a), ctx).unsqueeze(1)
-        vis = torch.arange(ctx).unsqueeze(0) <= qpos
+        kpos = torch.arange(ctx).unsqueeze(0)
+        vis = kpos <= qpos
+        if chunk > 0:
+            vis = vis & (kpos // chunk == qpos // chunk)
         sc = sc.masked_fill(~vis.unsqueeze(0), float("-inf"))
-        out[a:b] = torch.matmul(torch.softmax(sc, dim=-1), V).transpose(0, 1)
+        if sink is None:
+            w = torch.softmax(sc, dim=-1)
+        else:
+            # one more term exp(sink) in the denominator, no key, no value
+            sk = sink.float().view(heads, 1, 1)
+            m = torch.maximum(sc.max(-1, keepdim=True).values, sk)
+            e = torch.exp(sc - m)
+            w = e / (e.sum(-1, keepdim=True) + torch.exp(sk - m))
+        o = torch.matmul(w, V).transpose(0, 1)  # [n, heads, DV]
+        if out_inv_freq is not None:
+            # turn every head output back by its own position
+            o = rotate_halves(o, qpos.view(-1), out_inv_freq, -1.0)
+        out[a:b] = o
     if gate is not None:
         out = out * torch.sigmoid(gate.float()).unsqueeze(-1)
     return out.reshape(T, heads * DV).to(out_dtype)
+
+
+def rotary_inv_freq(n_rot: int, base: float) -> torch.Tensor:
+    """inv_freq[i] = base^(-2i/n_rot), i < n_rot/2, rounded once from float64."""
+    i = torch.arange(n_rot // 2, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / n_rot)).to(torch.float32)
+
+
+def rotate_halves(x, positions, inv_freq, sign: float = 1.0):
+    """Rotate the first 2*len(inv_freq) coordinates of the last axis of
+    x [T, heads, D] (fp32): coordinate i pairs with i + half, pair i turns by
+    sign * position * inv_freq[i]; angles and sin/cos in fp32."""
+    half = inv_freq.numel()
+    if half == 0:
+        return x
+    a = positions.to(torch.float32).view(-1, 1, 1) * inv_freq.view(1, 1, -1)
+    c, s = torch.cos(a), torch.sin(a) * sign
+    u, v = x[..., :half], x[..., half : 2 * half]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., 2 * half :]], dim=-1)
+
+
+def qk_headnorm_rope_cache(
+    q, k, v, qw, kw, positions, slot_mapping, k_cache, v_cache, eps,
+    heads: int, qk_inv_freq, v_unit_norm: bool, v_inv_freq,
+):
+    """Per-head RMS norm of q and k (weights [dim], shared by the heads),
+    rotary positions on their first 2*len(qk_inv_freq) coordinates; values
+    optionally divided by their per-head RMS and rotated by their position
+    over 2*len(v_inv_freq) coordinates; k / v scattered to the pages; q
+    returned in fp32."""
+    _, G, bs, D = k_cache.shape
+    DV = v_cache.shape[3]
+    T = q.shape[0]
+    qf = q.float().reshape(T, heads, D)
+    kf = k.float().reshape(T, G, D)
+    vf = v.float().reshape(T, G, DV)
+    qn = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps) * qw
+    kn = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps) * kw
+    if qk_inv_freq is not None:
+        qn = rotate_halves(qn, positions, qk_inv_freq)
+        kn = rotate_halves(kn, positions, qk_inv_freq)
+    if v_unit_norm:
+        vf = vf * torch.rsqrt(vf.pow(2).mean(-1, keepdim=True) + eps)
+    if v_inv_freq is not None:
+        vf = rotate_halves(vf, positions, v_inv_freq)
+    slots = slot_mapping.long()
+    ok = slots >= 0
+    blk, off = slots[ok] // bs, slots[ok] % bs
+    k_cache[blk, :, off] = kn[ok].to(k_cache.dtype)
+    v_cache[blk, :, off] = vf[ok].to(v_cache.dtype)
+    return qn.reshape(T, heads * D)
+
+
+def post_norm_add_rms_norm(
+    residual, delta, post_gain: float, layer_scale, eps: float,
+    next_gain: float, out_dtype, add_rows=None, add_vec=None,
+    want_out: bool = True,
+):
+    """residual (fp32, in place) += layer_scale * (delta / rms(delta) *
+    post_gain), then += add_rows (per token) and += add_vec (one row for
+    all) when given; returns residual / rms(residual) * next_gain in
+    ``out_dtype`` (None when ``want_out`` is false). Gains are scalars."""
+    if delta is not None:
+        d = delta.float()
+        d = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * post_gain
+        residual += d * layer_scale
+    if add_rows is not None:
+        residual += add_rows
+    if add_vec is not None:
+        residual += add_vec
+    if not want_out:
+        return None
+    inv = torch.rsqrt(residual.pow(2).mean(-1, keepdim=True) + eps)
+    return (residual * inv * next_gain).to(out_dtype)
+
+
+def router_topk(
+    logits, top: int, softmax: bool = False, renorm: bool = False,
+    dense: bool = False,
+):
+    """Scores (sigmoid, or softmax over the experts) of fp32 router logits
+    [T, E]; the ``top`` largest per token -> (indices int32 [T, top],
+    weights fp32 [T, top], and with ``dense`` the same weights as a [T, E]
+    matrix that is zero elsewhere), optionally renormalised to sum 1."""
+    z = logits.float()
+    s = torch.softmax(z, dim=-1) if softmax else torch.sigmoid(z)
+    w, idx = s.topk(top, dim=-1)
+    if renorm:
+        w = w / w.sum(-1, keepdim=True)
+    dw = torch.zeros_like(s).scatter_(1, idx, w) if dense else None
+    return idx.to(torch.int32), w, dw
+
+
+def route_tokens(
+    h, router, top: int, softmax: bool = False, renorm: bool = False,
+    dense: bool = False, want_logits: bool = False,
+):
+    """Router logits h @ router^T in fp32 (h in the activation dtype, router
+    fp32 [E, W]) followed by ``router_topk``; returns (indices, weights,
+    dense weights or None, logits or None)."""
+    logits = torch.nn.functional.linear(h.float(), router.float())
+    idx, w, dw = router_topk(logits, top, softmax, renorm, dense)
+    return idx, w, dw, (logits if want_logits else None)
+
+
+def gather_scale_rows(x, rows, scales):
+    """out[r] = x[rows[r]] * scales[r] (product in fp32, rounded to x's dtype)."""
+    return (x[rows.long()].float() * scales.float().unsqueeze(1)).to(x.dtype)
+
+
+def combine_rows(y, index, top: int, extra=None):
+    """out[t] = sum_k y[index[t * top + k]] (+ extra[t]), summed in fp32 in
+    the order k = 0..top-1, extra last; fp32 result."""
+    T = index.numel() // top
+    out = torch.zeros(T, y.shape[1], dtype=torch.float32, device=y.device)
+    idx = index.long().view(T, top)
+    for k in range(top):
+        out += y[idx[:, k]].float()
+    if extra is not None:
+        out += extra.float()
+    return out
 
 
 def clamped_swiglu(x, alpha: float, limit: float):
