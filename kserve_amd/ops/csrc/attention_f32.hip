@@ -6,6 +6,12 @@
 //    scale the query by a position-dependent temperature
 //        1 + coef * ln(floor((pos + 1) / every) + 1),
 //    write q (fp32) out and scatter k / v into the paged cache.
+//  * qk_headnorm_rope_cache: per token and per HEAD, RMS-normalise q and k
+//    with a weight of the head size shared by the heads, rotate the first
+//    2*half coordinates (coordinate i pairs with i + half, angle
+//    pos * inv_freq[i] in fp32), optionally divide each value head by its
+//    RMS and rotate it by the token's position over its whole width, write
+//    q (fp32) out and scatter k / v into the paged cache.
 //  * ctx_attention_f32: causal attention of a flat variable-length query
 //    batch against each sequence's pages (the portion's own keys are already
 //    in the cache). Both products run on the fp32 matrix cores
@@ -19,6 +25,12 @@
 //    order; V is read from LDS in that order), so the weights never leave
 //    registers. The head-dimension contraction and the value columns are
 //    likewise assigned to lanes so that every LDS operand read is 16 bytes.
+//    Optional parts: a chunk-local mask (a query sees only keys of its own
+//    block of `chunk` positions, so the key loop starts at the chunk of the
+//    block's first query), a per-head sink (one more term exp(sink) in the
+//    softmax denominator, with no key and no value), and turning every
+//    head output back by its query's position (pairs m, m + DV/2; the
+//    normalised rows pass through LDS so a pair meets in one lane).
 //    Prefill: a block takes 64 consecutive tokens of one query head, 16 per
 //    wave, all waves sharing the staged K/V tile. Decode (one token per
 //    sequence): a block takes the query heads of one KV group as its 16
@@ -81,6 +93,153 @@ __global__ void qk_norm_temp_cache_kernel(
   for (int i = threadIdx.x; i < kv_heads * DV; i += NT) {
     const int g = i / DV, d = i % DV;
     v_cache[((blk * kv_heads + g) * block_size + off) * DV + d] = vr[i];
+  }
+}
+
+// A block per token. The angles depend on the token's position only, so
+// their sines and cosines are computed once per block into LDS ([qk_half]
+// then [v_half] pairs) and shared by every head. Then one wave per head
+// job: jobs 0..heads-1 are q heads, then kv_heads k heads, then kv_heads v
+// heads. x_n[j] = x[j] * inv_rms * w[j]; coordinate i < half pairs with
+// i + half. VEC = 2: a lane owns two neighbouring coordinates (4- and 8-byte
+// accesses); needs even head sizes, halves and row stride.
+template <int VEC>
+__device__ __forceinline__ void ld_vec(const short* p, float* v) {
+  if (VEC == 2) {
+    const unsigned u = *reinterpret_cast<const unsigned*>(p);
+    v[0] = bf16_bits_to_float((short)(u & 0xffffu));
+    v[1] = bf16_bits_to_float((short)(u >> 16));
+  } else {
+    v[0] = bf16_bits_to_float(p[0]);
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void ld_vec(const float* p, float* v) {
+  if (VEC == 2) {
+    const float2_t u = *reinterpret_cast<const float2_t*>(p);
+    v[0] = u[0];
+    v[1] = u[1];
+  } else {
+    v[0] = p[0];
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void st_vec(short* p, const float* v) {
+  if (VEC == 2) {
+    const unsigned lo = (unsigned short)float_to_bf16_bits(v[0]);
+    const unsigned hi = (unsigned short)float_to_bf16_bits(v[1]);
+    *reinterpret_cast<unsigned*>(p) = lo | (hi << 16);
+  } else {
+    p[0] = float_to_bf16_bits(v[0]);
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void st_vec(float* p, const float* v) {
+  if (VEC == 2)
+    *reinterpret_cast<float2_t*>(p) = float2_t{v[0], v[1]};
+  else
+    p[0] = v[0];
+}
+
+template <typename T, int VEC>
+__global__ void qk_headnorm_rope_cache_kernel(
+    float* __restrict__ q_out, const T* __restrict__ q, const T* __restrict__ k,
+    const T* __restrict__ v, long row_stride, const float* __restrict__ qw,
+    const float* __restrict__ kw, const long* __restrict__ positions,
+    const int* __restrict__ slot_mapping, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, float eps, int heads, int kv_heads, int D, int DV,
+    int block_size, const float* __restrict__ qk_inv_freq, int qk_half,
+    int v_unit_norm, const float* __restrict__ v_inv_freq, int v_half) {
+  extern __shared__ float lds[];
+  if (!qk_inv_freq) qk_half = 0;
+  if (!v_inv_freq) v_half = 0;
+  float* cs_qk = lds;               // [qk_half][2] = (cos, sin)
+  float* cs_v = lds + 2 * qk_half;  // [v_half][2]
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const float pos = (float)positions[t];
+  for (int i = threadIdx.x; i < qk_half + v_half; i += NT) {
+    const float f = i < qk_half ? qk_inv_freq[i] : v_inv_freq[i - qk_half];
+    float sn, cs;
+    sincosf(pos * f, &sn, &cs);
+    lds[2 * i] = cs;
+    lds[2 * i + 1] = sn;
+  }
+  __syncthreads();
+  const long slot = slot_mapping[t];
+  const long blk = slot >= 0 ? slot / block_size : 0;
+  const long off = slot >= 0 ? slot % block_size : 0;
+  const int jobs = heads + 2 * kv_heads;
+  for (int job = wave; job < jobs; job += NW) {
+    const T* src;
+    const float* w = nullptr;
+    const float* cs;
+    int width, half;
+    bool norm = true;
+    float* dst_f = nullptr;
+    T* dst_c = nullptr;
+    if (job < heads) {
+      src = q + t * row_stride + (long)job * D;
+      w = qw;
+      width = D;
+      cs = cs_qk;
+      half = qk_half;
+      dst_f = q_out + (t * heads + job) * D;
+    } else if (job < heads + kv_heads) {
+      const int g = job - heads;
+      src = k + t * row_stride + (long)g * D;
+      w = kw;
+      width = D;
+      cs = cs_qk;
+      half = qk_half;
+      if (slot < 0) continue;
+      dst_c = k_cache + ((blk * kv_heads + g) * block_size + off) * D;
+    } else {
+      const int g = job - heads - kv_heads;
+      src = v + t * row_stride + (long)g * DV;
+      width = DV;
+      cs = cs_v;
+      half = v_half;
+      norm = v_unit_norm != 0;
+      if (slot < 0) continue;
+      dst_c = v_cache + ((blk * kv_heads + g) * block_size + off) * DV;
+    }
+    float inv = 1.0f;
+    if (norm) {
+      float ss = 0.f;
+      for (int i = lane * VEC; i < width; i += WAVE_SIZE * VEC) {
+        float x[VEC];
+        ld_vec<VEC>(src + i, x);
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) ss += x[c] * x[c];
+      }
+      ss = wave_reduce_sum(ss);
+      inv = 1.0f / sqrtf(ss / (float)width + eps);
+    }
+    for (int i = lane * VEC; i < width; i += WAVE_SIZE * VEC) {
+      float x[VEC], r[VEC];
+      ld_vec<VEC>(src + i, x);
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) {
+        if (norm) x[c] = w ? x[c] * inv * w[i + c] : x[c] * inv;
+        r[c] = x[c];
+      }
+      if (i < 2 * half) {  // i and i + VEC - 1 lie in the same half
+        const int pi = i < half ? i + half : i - half;  // partner
+        const int fi = i < half ? i : i - half;
+        float y[VEC];
+        ld_vec<VEC>(src + pi, y);
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+          if (norm) y[c] = w ? y[c] * inv * w[pi + c] : y[c] * inv;
+          const float co = cs[2 * (fi + c)], sn = cs[2 * (fi + c) + 1];
+          r[c] = i < half ? x[c] * co - y[c] * sn : x[c] * co + y[c] * sn;
+        }
+      }
+      if (dst_f) st_vec<VEC>(dst_f + i, r);
+      else st_vec<VEC>(dst_c + i, r);
+    }
   }
 }
 
@@ -178,7 +337,9 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
     const T* __restrict__ gate, long gate_stride, float scale, int heads,
-    int kv_heads, int D, int DV, int block_size, int hpb) {
+    int kv_heads, int D, int DV, int block_size, int hpb,
+    const float* __restrict__ sink, int chunk,
+    const float* __restrict__ out_inv_freq) {
   extern __shared__ float lds[];
   constexpr int KS = DP + 4;   // K row stride: lanes of one MFMA read hit 64 banks
   constexpr int VS = DVP + 4;  // V row stride: likewise for the 4-key-apart rows
@@ -211,9 +372,17 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   const int tok = q0 + tok0 + r / hpb;
   const int hd = head0 + r % hpb;
   const int qpos = row_ok ? base_pos + r / hpb : -1;
-  // keys this wave needs: up to its own last row's position
+  // first visible key of this lane's query, of the block and of this wave
+  const int qstart = (chunk > 0 && row_ok) ? qpos / chunk * chunk : 0;
+  const int kbeg = chunk > 0 ? base_pos / chunk * chunk : 0;
+  // keys this wave needs: from its first row's chunk up to its own last
+  // row's position
   const int wave_last =
       SPLITK ? last_pos : base_pos + min(wave * 16 + 15, nrows - 1) / hpb;
+  const int wave_first =
+      (SPLITK || chunk <= 0)
+          ? kbeg
+          : (base_pos + min(wave * 16, nrows - 1) / hpb) / chunk * chunk;
 
   // Q^T fragments (B operand). The contraction over the head dimension may
   // run in any order as long as both operands agree: k-step ks of lane group
@@ -241,9 +410,9 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   // the next tile's global loads are in flight while this one is computed
   TileStage<T, DP> kst;
   TileStage<T, DVP> vst;
-  kst.fetch(k_cache, bt, 0, min(BK, last_pos + 1), g, kv_heads, D, block_size, bs_shift, kvec);
-  vst.fetch(v_cache, bt, 0, min(BK, last_pos + 1), g, kv_heads, DV, block_size, bs_shift, vvec);
-  for (int k0 = 0; k0 <= last_pos; k0 += BK) {
+  kst.fetch(k_cache, bt, kbeg, min(BK, last_pos + 1 - kbeg), g, kv_heads, D, block_size, bs_shift, kvec);
+  vst.fetch(v_cache, bt, kbeg, min(BK, last_pos + 1 - kbeg), g, kv_heads, DV, block_size, bs_shift, vvec);
+  for (int k0 = kbeg; k0 <= last_pos; k0 += BK) {
     __syncthreads();  // previous tile fully consumed
     kst.store(Ks);
     vst.store(Vs);
@@ -253,7 +422,7 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
       kst.fetch(k_cache, bt, k0 + BK, nn, g, kv_heads, D, block_size, bs_shift, kvec);
       vst.fetch(v_cache, bt, k0 + BK, nn, g, kv_heads, DV, block_size, bs_shift, vvec);
     }
-    if (k0 > wave_last) continue;
+    if (k0 > wave_last || k0 + BK <= wave_first) continue;
 
     // S^T sub-tiles: acc[kt][v] = score(key k0 + 16 kt' + 4 lg + v, query li)
     // k-steps outermost, two accumulators per sub-tile: 2 KT independent
@@ -286,7 +455,7 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int kp = k0 + 16 * kt + 4 * lg + v;
-        sc[t][v] = kp <= qpos ? sc[t][v] : -INFINITY;
+        sc[t][v] = (kp <= qpos && kp >= qstart) ? sc[t][v] : -INFINITY;
         mt = fmaxf(mt, sc[t][v]);
       }
     }
@@ -348,37 +517,89 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
       for (int v = 0; v < 4; ++v)
         Os[(wave * 16 + li) * DVP + 64 * (i / 4) + 4 * (4 * lg + v) + i % 4] = o[i][v];
     __syncthreads();
-    for (int e = threadIdx.x; e < nrows * DVP; e += NT) {
-      const int row = e / DVP, dv = e % DVP;
-      if (dv >= DV) continue;
+    // an element pair (dv, dv + DV/2) per thread when the output is turned
+    // back, else one element
+    const int ohalf = out_inv_freq ? DV / 2 : 0;
+    const int per_row = out_inv_freq ? ohalf : DV;
+    for (int e = threadIdx.x; e < nrows * per_row; e += NT) {
+      const int row = e / per_row, dv = e % per_row;
+      const int tk = q0 + tok0 + row / hpb, h2 = head0 + row % hpb;
       float M = -INFINITY;
 #pragma unroll
       for (int w = 0; w < NW; ++w) M = fmaxf(M, Ms[w * 16 + row]);
-      float L = 0.f, O = 0.f;
+      float L = 0.f;
+      if (sink) {
+        const float sl = sink[h2] * 1.44269504088896340736f;
+        M = fmaxf(M, sl);
+        L = exp2f(sl - M);
+      }
+      float O = 0.f, O2 = 0.f;
 #pragma unroll
       for (int w = 0; w < NW; ++w) {
         const float mw = Ms[w * 16 + row];
         const float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
         L += Ls[w * 16 + row] * f;
         O += Os[(w * 16 + row) * DVP + dv] * f;
+        if (out_inv_freq) O2 += Os[(w * 16 + row) * DVP + dv + ohalf] * f;
       }
-      const int tk = q0 + tok0 + row / hpb, h2 = head0 + row % hpb;
       float f = 1.0f / L;
       if (gate) {
         const float gv = ld_f32(gate, (long)tk * gate_stride + h2);
         f *= 1.0f / (1.0f + expf(-gv));
       }
-      st_f32(out, ((long)tk * heads + h2) * DV + dv, O * f);
+      O *= f;
+      if (out_inv_freq) {
+        O2 *= f;
+        float sn, cs;
+        sincosf((float)(base_pos + row / hpb) * out_inv_freq[dv], &sn, &cs);
+        st_f32(out, ((long)tk * heads + h2) * DV + dv, O * cs + O2 * sn);
+        st_f32(out, ((long)tk * heads + h2) * DV + dv + ohalf, O2 * cs - O * sn);
+      } else {
+        st_f32(out, ((long)tk * heads + h2) * DV + dv, O);
+      }
     }
     return;
   }
 
-  if (!row_ok) return;
-  float f = 1.0f / l;
-  if (gate) {
+  if (row_ok && sink) {
+    const float sl = sink[hd] * 1.44269504088896340736f;
+    const float mn = fmaxf(m, sl);
+    const float corr = m == -INFINITY ? 0.f : exp2f(m - mn);
+    l = l * corr + exp2f(sl - mn);
+#pragma unroll
+    for (int i = 0; i < DVP / 16; ++i) o[i] *= corr;
+  }
+  float f = row_ok ? 1.0f / l : 0.f;
+  if (row_ok && gate) {
     const float gv = ld_f32(gate, (long)tok * gate_stride + hd);
     f *= 1.0f / (1.0f + expf(-gv));
   }
+  if (out_inv_freq) {
+    // rows through LDS [64][DVP + 1] so that a lane holds both halves of a pair
+    constexpr int OS = DVP + 1;
+    __syncthreads();  // every wave is done with the K/V tiles
+    float* Os = lds;
+    if (row_ok) {
+#pragma unroll
+      for (int i = 0; i < DVP / 16; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          Os[r * OS + 64 * (i / 4) + 4 * (4 * lg + v) + i % 4] = o[i][v] * f;
+    }
+    __syncthreads();
+    const int ohalf = DV / 2;
+    for (int e = threadIdx.x; e < nrows * ohalf; e += NT) {
+      const int row = e / ohalf, dv = e % ohalf;
+      const int tk = q0 + tok0 + row / hpb, h2 = head0 + row % hpb;
+      const float a = Os[row * OS + dv], b = Os[row * OS + dv + ohalf];
+      float sn, cs;
+      sincosf((float)(base_pos + row / hpb) * out_inv_freq[dv], &sn, &cs);
+      st_f32(out, ((long)tk * heads + h2) * DV + dv, a * cs + b * sn);
+      st_f32(out, ((long)tk * heads + h2) * DV + dv + ohalf, b * cs - a * sn);
+    }
+    return;
+  }
+  if (!row_ok) return;
 #pragma unroll
   for (int i = 0; i < DVP / 16; ++i)
 #pragma unroll
@@ -417,6 +638,47 @@ extern "C" hipError_t ks_qk_norm_temp_cache(
   return hipSuccess;
 }
 
+extern "C" hipError_t ks_qk_headnorm_rope_cache(
+    void* q_out, const void* q, const void* k, const void* v, long row_stride,
+    const void* qw, const void* kw, const void* positions,
+    const void* slot_mapping, void* k_cache, void* v_cache, float eps,
+    int tokens, int heads, int kv_heads, int D, int DV, int block_size,
+    const void* qk_inv_freq, int qk_half, int v_unit_norm,
+    const void* v_inv_freq, int v_half, int is_f32, hipStream_t stream) {
+  if (tokens == 0) return hipSuccess;
+  if (2 * qk_half > D || 2 * v_half > DV) return hipErrorInvalidValue;
+#define HN_ARGS(TT)                                                          \
+  (float*)q_out, (const TT*)q, (const TT*)k, (const TT*)v, row_stride,       \
+      (const float*)qw, (const float*)kw, (const long*)positions,            \
+      (const int*)slot_mapping, (TT*)k_cache, (TT*)v_cache, eps, heads,      \
+      kv_heads, D, DV, block_size, (const float*)qk_inv_freq, qk_half,       \
+      v_unit_norm, (const float*)v_inv_freq, v_half
+  const size_t smem = sizeof(float) * 2 * (size_t)(qk_half + v_half);
+  const int esz = is_f32 ? 4 : 2;
+  auto al = [&](const void* p) { return ((uintptr_t)p % (2 * esz)) == 0; };
+  const bool vec = D % 2 == 0 && DV % 2 == 0 && qk_half % 2 == 0 &&
+                   v_half % 2 == 0 && row_stride % 2 == 0 && al(q) && al(k) &&
+                   al(v) && al(k_cache) && al(v_cache) &&
+                   ((uintptr_t)q_out % 8) == 0;
+  if (is_f32) {
+    if (vec)
+      hipLaunchKernelGGL((qk_headnorm_rope_cache_kernel<float, 2>), dim3(tokens),
+                         dim3(NT), smem, stream, HN_ARGS(float));
+    else
+      hipLaunchKernelGGL((qk_headnorm_rope_cache_kernel<float, 1>), dim3(tokens),
+                         dim3(NT), smem, stream, HN_ARGS(float));
+  } else {
+    if (vec)
+      hipLaunchKernelGGL((qk_headnorm_rope_cache_kernel<short, 2>), dim3(tokens),
+                         dim3(NT), smem, stream, HN_ARGS(short));
+    else
+      hipLaunchKernelGGL((qk_headnorm_rope_cache_kernel<short, 1>), dim3(tokens),
+                         dim3(NT), smem, stream, HN_ARGS(short));
+  }
+  HIP_CHECK_KERNEL();
+  return hipSuccess;
+}
+
 template <typename T, int DP, int DVP>
 hipError_t launch_ctx_attention(void* out, const void* q, const void* k_cache,
                                 const void* v_cache, const void* block_tables,
@@ -424,7 +686,9 @@ hipError_t launch_ctx_attention(void* out, const void* q, const void* k_cache,
                                 const void* ctx_lens, const void* gate,
                                 long gate_stride, float scale, int num_seqs,
                                 int max_q_len, int heads, int kv_heads, int D,
-                                int DV, int block_size, hipStream_t stream) {
+                                int DV, int block_size, const void* sink,
+                                int chunk, const void* out_inv_freq,
+                                hipStream_t stream) {
   size_t smem = sizeof(float) * (size_t)BK * (DP + 4 + DVP + 4);
   const bool decode = max_q_len == 1;
   // decode: one token per sequence, a block takes heads of one group
@@ -449,14 +713,15 @@ hipError_t launch_ctx_attention(void* out, const void* q, const void* k_cache,
                      (const T*)k_cache, (const T*)v_cache,
                      (const int*)block_tables, bt_stride, (const int*)cu_q,
                      (const int*)ctx_lens, (const T*)gate, gate_stride, scale,
-                     heads, kv_heads, D, DV, block_size, hpb);
+                     heads, kv_heads, D, DV, block_size, hpb,
+                     (const float*)sink, chunk, (const float*)out_inv_freq);
   return hipGetLastError();
 }
 
 #define CTX_ARGS                                                              \
   out, q, k_cache, v_cache, block_tables, bt_stride, cu_q, ctx_lens, gate,    \
       gate_stride, scale, num_seqs, max_q_len, heads, kv_heads, D, DV,        \
-      block_size, stream
+      block_size, sink, chunk, out_inv_freq, stream
 
 template <typename T, int DP>
 hipError_t dispatch_dv(void* out, const void* q, const void* k_cache,
@@ -464,7 +729,9 @@ hipError_t dispatch_dv(void* out, const void* q, const void* k_cache,
                        int bt_stride, const void* cu_q, const void* ctx_lens,
                        const void* gate, long gate_stride, float scale,
                        int num_seqs, int max_q_len, int heads, int kv_heads,
-                       int D, int DV, int block_size, hipStream_t stream) {
+                       int D, int DV, int block_size, const void* sink,
+                       int chunk, const void* out_inv_freq,
+                       hipStream_t stream) {
   if (DV <= 64) return launch_ctx_attention<T, DP, 64>(CTX_ARGS);
   if (DV <= 128) return launch_ctx_attention<T, DP, 128>(CTX_ARGS);
   return launch_ctx_attention<T, DP, 256>(CTX_ARGS);
@@ -476,7 +743,9 @@ hipError_t dispatch_d(void* out, const void* q, const void* k_cache,
                       int bt_stride, const void* cu_q, const void* ctx_lens,
                       const void* gate, long gate_stride, float scale,
                       int num_seqs, int max_q_len, int heads, int kv_heads,
-                      int D, int DV, int block_size, hipStream_t stream) {
+                      int D, int DV, int block_size, const void* sink,
+                      int chunk, const void* out_inv_freq,
+                      hipStream_t stream) {
   if (D <= 64) return dispatch_dv<T, 64>(CTX_ARGS);
   if (D <= 128) return dispatch_dv<T, 128>(CTX_ARGS);
   return dispatch_dv<T, 256>(CTX_ARGS);
@@ -487,10 +756,11 @@ extern "C" hipError_t ks_ctx_attention_f32(
     const void* block_tables, int bt_stride, const void* cu_q,
     const void* ctx_lens, const void* gate, long gate_stride, float scale,
     int num_seqs, int max_q_len, int heads, int kv_heads, int D, int DV,
-    int block_size, int is_f32, hipStream_t stream) {
+    int block_size, int is_f32, const void* sink, int chunk,
+    const void* out_inv_freq, hipStream_t stream) {
   if (num_seqs == 0 || max_q_len == 0) return hipSuccess;
   if (D < 1 || D > 256 || DV < 1 || DV > 256 || kv_heads < 1 ||
-      heads % kv_heads != 0)
+      heads % kv_heads != 0 || chunk < 0 || (out_inv_freq && DV % 2 != 0))
     return hipErrorInvalidValue;
   return is_f32 ? dispatch_d<float>(CTX_ARGS) : dispatch_d<short>(CTX_ARGS);
 }

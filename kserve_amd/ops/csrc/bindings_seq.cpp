@@ -30,7 +30,27 @@ hipError_t ks_qk_norm_temp_cache(void*, const void*, const void*, const void*,
 hipError_t ks_ctx_attention_f32(void*, const void*, const void*, const void*,
                                 const void*, int, const void*, const void*,
                                 const void*, long, float, int, int, int, int,
-                                int, int, int, int, hipStream_t);
+                                int, int, int, int, const void*, int,
+                                const void*, hipStream_t);
+hipError_t ks_qk_headnorm_rope_cache(void*, const void*, const void*,
+                                     const void*, long, const void*,
+                                     const void*, const void*, const void*,
+                                     void*, void*, float, int, int, int, int,
+                                     int, int, const void*, int, int,
+                                     const void*, int, int, hipStream_t);
+hipError_t ks_post_norm_add_rms_norm(void*, const void*, long, int, float,
+                                     const void*, const void*, const void*,
+                                     float, float, void*, int, int, int,
+                                     hipStream_t);
+hipError_t ks_router_topk(void*, void*, void*, const void*, int, int, int, int,
+                          int, hipStream_t);
+hipError_t ks_route_tokens(void*, void*, void*, void*, const void*, long,
+                           const void*, int, int, int, int, int, int, int,
+                           hipStream_t);
+hipError_t ks_gather_scale_rows(void*, const void*, long, const void*,
+                                const void*, int, int, int, hipStream_t);
+hipError_t ks_combine_rows(void*, const void*, const void*, int, const void*,
+                           long, int, int, int, hipStream_t);
 hipError_t ks_clamped_swiglu(void*, const void*, int, int, float, float, int,
                              hipStream_t);
 }
@@ -62,20 +82,28 @@ int act_is_f32(const at::Tensor& t, const char* name) {
   TORCH_CHECK((t).dim() == 2 && (t).stride(1) == 1, #t " rows must be dense")
 
 void embed_scale_sinpos(at::Tensor& out, at::Tensor& table, at::Tensor& tokens,
-                        at::Tensor& positions, at::Tensor& inv_freq,
+                        at::Tensor& positions,
+                        const c10::optional<at::Tensor>& inv_freq_opt,
                         double scale) {
   CHECK_F32(out);
-  CHECK_F32(inv_freq);
+  const void* inv_freq_ptr = nullptr;
+  int64_t n_freq = 1 << 30;
+  if (inv_freq_opt.has_value()) {
+    const at::Tensor& inv_freq = *inv_freq_opt;
+    CHECK_F32(inv_freq);
+    inv_freq_ptr = inv_freq.data_ptr();
+    n_freq = inv_freq.numel();
+  }
   CHECK_I64(tokens);
   CHECK_I64(positions);
   TORCH_CHECK(table.is_contiguous() && table.dim() == 2, "table [vocab, width]");
   const int width = table.size(1), rows = tokens.numel();
   TORCH_CHECK(out.numel() == (int64_t)rows * width &&
-                  positions.numel() == rows && inv_freq.numel() * 2 >= width,
+                  positions.numel() == rows && n_freq * 2 >= width,
               "embed_scale_sinpos: shape mismatch");
   check_hip(ks_embed_scale_sinpos(out.data_ptr(), table.data_ptr(),
                                   tokens.data_ptr(), positions.data_ptr(),
-                                  inv_freq.data_ptr(), (float)scale, rows,
+                                  inv_freq_ptr, (float)scale, rows,
                                   width, act_is_f32(table, "table"),
                                   current_stream()),
             "embed_scale_sinpos");
@@ -256,7 +284,9 @@ void ctx_attention_f32(at::Tensor& out, at::Tensor& q, at::Tensor& k_cache,
                        at::Tensor& v_cache, at::Tensor& block_tables,
                        at::Tensor& cu_q, at::Tensor& ctx_lens,
                        const c10::optional<at::Tensor>& gate, double scale,
-                       int64_t max_q_len, int64_t heads) {
+                       int64_t max_q_len, int64_t heads,
+                       const c10::optional<at::Tensor>& sink, int64_t chunk,
+                       const c10::optional<at::Tensor>& out_inv_freq) {
   CHECK_F32(q);
   CHECK_I32(cu_q);
   CHECK_I32(ctx_lens);
@@ -290,14 +320,234 @@ void ctx_attention_f32(at::Tensor& out, at::Tensor& q, at::Tensor& k_cache,
     gp = gate->data_ptr();
     gst = gate->stride(0);
   }
+  const void *sp = nullptr, *fp = nullptr;
+  if (sink.has_value()) {
+    CHECK_F32(*sink);
+    TORCH_CHECK(sink->numel() == heads, "sink [heads] fp32");
+    sp = sink->data_ptr();
+  }
+  if (out_inv_freq.has_value()) {
+    CHECK_F32(*out_inv_freq);
+    TORCH_CHECK(DV % 2 == 0 && out_inv_freq->numel() == DV / 2,
+                "out_inv_freq [vdim / 2] fp32");
+    fp = out_inv_freq->data_ptr();
+  }
+  TORCH_CHECK(chunk >= 0, "chunk must not be negative");
   check_hip(ks_ctx_attention_f32(
                 out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
                 v_cache.data_ptr(), block_tables.data_ptr(),
                 (int)block_tables.stride(0), cu_q.data_ptr(),
                 ctx_lens.data_ptr(), gp, gst, (float)scale, num_seqs,
-                (int)max_q_len, (int)heads, G, D, DV, bs, f32,
-                current_stream()),
+                (int)max_q_len, (int)heads, G, D, DV, bs, f32, sp, (int)chunk,
+                fp, current_stream()),
             "ctx_attention_f32");
+}
+
+void qk_headnorm_rope_cache(at::Tensor& q_out, at::Tensor& q, at::Tensor& k,
+                            at::Tensor& v, at::Tensor& qw, at::Tensor& kw,
+                            at::Tensor& positions, at::Tensor& slot_mapping,
+                            at::Tensor& k_cache, at::Tensor& v_cache,
+                            double eps, int64_t heads,
+                            const c10::optional<at::Tensor>& qk_inv_freq,
+                            bool v_unit_norm,
+                            const c10::optional<at::Tensor>& v_inv_freq) {
+  CHECK_F32(q_out);
+  CHECK_F32(qw);
+  CHECK_F32(kw);
+  CHECK_ROWS(q);
+  CHECK_ROWS(k);
+  CHECK_ROWS(v);
+  CHECK_I64(positions);
+  CHECK_I32(slot_mapping);
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 &&
+                  k_cache.is_contiguous() && v_cache.is_contiguous(),
+              "caches [blocks, kv_heads, block, dim]");
+  const int f32 = act_is_f32(q, "q");
+  const int tokens = q.size(0);
+  const int G = k_cache.size(1), bs = k_cache.size(2), D = k_cache.size(3);
+  const int DV = v_cache.size(3);
+  TORCH_CHECK(act_is_f32(k, "k") == f32 && act_is_f32(v, "v") == f32 &&
+                  act_is_f32(k_cache, "k_cache") == f32 &&
+                  act_is_f32(v_cache, "v_cache") == f32,
+              "qk_headnorm_rope_cache: dtype mismatch");
+  TORCH_CHECK(q.size(1) == heads * D && k.size(1) == G * D &&
+                  v.size(1) == G * DV && k.size(0) == tokens &&
+                  v.size(0) == tokens && q.stride(0) == k.stride(0) &&
+                  q.stride(0) == v.stride(0) && qw.numel() == D &&
+                  kw.numel() == D && v_cache.size(1) == G &&
+                  v_cache.size(2) == bs && v_cache.size(0) == k_cache.size(0) &&
+                  q_out.numel() == (int64_t)tokens * heads * D &&
+                  positions.numel() >= tokens && slot_mapping.numel() >= tokens,
+              "qk_headnorm_rope_cache: shape mismatch");
+  const void *qf = nullptr, *vf = nullptr;
+  int qh = 0, vh = 0;
+  if (qk_inv_freq.has_value()) {
+    CHECK_F32(*qk_inv_freq);
+    qh = qk_inv_freq->numel();
+    TORCH_CHECK(2 * qh <= D, "more rotated coordinates than the head has");
+    qf = qk_inv_freq->data_ptr();
+  }
+  if (v_inv_freq.has_value()) {
+    CHECK_F32(*v_inv_freq);
+    vh = v_inv_freq->numel();
+    TORCH_CHECK(2 * vh <= DV, "more rotated coordinates than the value has");
+    vf = v_inv_freq->data_ptr();
+  }
+  check_hip(ks_qk_headnorm_rope_cache(
+                q_out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                q.stride(0), qw.data_ptr(), kw.data_ptr(),
+                positions.data_ptr(), slot_mapping.data_ptr(),
+                k_cache.data_ptr(), v_cache.data_ptr(), (float)eps, tokens,
+                (int)heads, G, D, DV, bs, qf, qh, v_unit_norm ? 1 : 0, vf, vh,
+                f32, current_stream()),
+            "qk_headnorm_rope_cache");
+}
+
+void post_norm_add_rms_norm(at::Tensor& residual,
+                            const c10::optional<at::Tensor>& delta,
+                            double post_gain,
+                            const c10::optional<at::Tensor>& layer_scale,
+                            double eps, double next_gain,
+                            const c10::optional<at::Tensor>& out,
+                            const c10::optional<at::Tensor>& add_rows,
+                            const c10::optional<at::Tensor>& add_vec) {
+  CHECK_F32(residual);
+  TORCH_CHECK(residual.dim() == 2, "residual [T, W]");
+  const int rows = residual.size(0), width = residual.size(1);
+  const void *dp = nullptr, *lp = nullptr, *rp = nullptr, *vp = nullptr;
+  void* op = nullptr;
+  long dst = 0;
+  int d_f32 = 1, o_f32 = 1;
+  if (delta.has_value()) {
+    CHECK_ROWS(*delta);
+    TORCH_CHECK(layer_scale.has_value(), "delta needs a layer scale");
+    CHECK_F32(*layer_scale);
+    TORCH_CHECK(delta->size(0) == rows && delta->size(1) == width &&
+                    layer_scale->numel() == width,
+                "delta / layer_scale: shape mismatch");
+    d_f32 = act_is_f32(*delta, "delta");
+    dp = delta->data_ptr();
+    dst = delta->stride(0);
+    lp = layer_scale->data_ptr();
+  }
+  if (add_rows.has_value()) {
+    CHECK_F32(*add_rows);
+    TORCH_CHECK(add_rows->numel() == residual.numel(), "add_rows [T, W]");
+    rp = add_rows->data_ptr();
+  }
+  if (add_vec.has_value()) {
+    CHECK_F32(*add_vec);
+    TORCH_CHECK(add_vec->numel() == width, "add_vec [W]");
+    vp = add_vec->data_ptr();
+  }
+  if (out.has_value()) {
+    TORCH_CHECK(out->is_contiguous() && out->numel() == residual.numel(),
+                "out [T, W]");
+    o_f32 = act_is_f32(*out, "out");
+    op = out->data_ptr();
+  }
+  check_hip(ks_post_norm_add_rms_norm(residual.data_ptr(), dp, dst, d_f32,
+                                      (float)post_gain, lp, rp, vp, (float)eps,
+                                      (float)next_gain, op, o_f32, rows, width,
+                                      current_stream()),
+            "post_norm_add_rms_norm");
+}
+
+void router_topk(at::Tensor& idx, at::Tensor& w,
+                 const c10::optional<at::Tensor>& dense, at::Tensor& logits,
+                 bool softmax, bool renorm) {
+  CHECK_F32(logits);
+  CHECK_F32(w);
+  CHECK_I32(idx);
+  TORCH_CHECK(logits.dim() == 2 && idx.dim() == 2, "logits [T, E], idx [T, top]");
+  const int T = logits.size(0), E = logits.size(1), top = idx.size(1);
+  TORCH_CHECK(idx.size(0) == T && w.numel() == idx.numel(),
+              "router_topk: shape mismatch");
+  void* dp = nullptr;
+  if (dense.has_value()) {
+    CHECK_F32(*dense);
+    TORCH_CHECK(dense->numel() == logits.numel(), "dense [T, E]");
+    dp = dense->data_ptr();
+  }
+  check_hip(ks_router_topk(idx.data_ptr(), w.data_ptr(), dp, logits.data_ptr(),
+                           T, E, top, softmax ? 1 : 0, renorm ? 1 : 0,
+                           current_stream()),
+            "router_topk");
+}
+
+void route_tokens(at::Tensor& idx, at::Tensor& w,
+                  const c10::optional<at::Tensor>& dense,
+                  const c10::optional<at::Tensor>& logits_out, at::Tensor& h,
+                  at::Tensor& router, bool softmax, bool renorm) {
+  CHECK_ROWS(h);
+  CHECK_F32(router);
+  CHECK_F32(w);
+  CHECK_I32(idx);
+  TORCH_CHECK(router.dim() == 2 && idx.dim() == 2,
+              "router [E, W], idx [T, top]");
+  const int T = h.size(0), W = h.size(1), E = router.size(0), top = idx.size(1);
+  TORCH_CHECK(router.size(1) == W && idx.size(0) == T &&
+                  w.numel() == idx.numel(),
+              "route_tokens: shape mismatch");
+  void *dp = nullptr, *lp = nullptr;
+  if (dense.has_value()) {
+    CHECK_F32(*dense);
+    TORCH_CHECK(dense->numel() == (int64_t)T * E, "dense [T, E]");
+    dp = dense->data_ptr();
+  }
+  if (logits_out.has_value()) {
+    CHECK_F32(*logits_out);
+    TORCH_CHECK(logits_out->numel() == (int64_t)T * E, "logits [T, E]");
+    lp = logits_out->data_ptr();
+  }
+  check_hip(ks_route_tokens(idx.data_ptr(), w.data_ptr(), dp, lp, h.data_ptr(),
+                            h.stride(0), router.data_ptr(), T, W, E, top,
+                            softmax ? 1 : 0, renorm ? 1 : 0,
+                            act_is_f32(h, "h"), current_stream()),
+            "route_tokens");
+}
+
+void gather_scale_rows(at::Tensor& out, at::Tensor& x, at::Tensor& rows,
+                       at::Tensor& scales) {
+  CHECK_ROWS(x);
+  CHECK_I32(rows);
+  CHECK_F32(scales);
+  const int f32 = act_is_f32(x, "x");
+  TORCH_CHECK(out.is_contiguous() && act_is_f32(out, "out") == f32 &&
+                  out.numel() == rows.numel() * x.size(1) &&
+                  scales.numel() == rows.numel(),
+              "gather_scale_rows: dtype/shape mismatch");
+  check_hip(ks_gather_scale_rows(out.data_ptr(), x.data_ptr(), x.stride(0),
+                                 rows.data_ptr(), scales.data_ptr(),
+                                 (int)rows.numel(), (int)x.size(1), f32,
+                                 current_stream()),
+            "gather_scale_rows");
+}
+
+void combine_rows(at::Tensor& out, at::Tensor& y, at::Tensor& index,
+                  int64_t top, const c10::optional<at::Tensor>& extra) {
+  CHECK_F32(out);
+  CHECK_I32(index);
+  TORCH_CHECK(y.dim() == 2 && y.is_contiguous() && top > 0 &&
+                  index.numel() % top == 0,
+              "y [rows, W] contiguous, index [T * top]");
+  const int f32 = act_is_f32(y, "y");
+  const int tokens = index.numel() / top, width = y.size(1);
+  TORCH_CHECK(out.numel() == (int64_t)tokens * width, "out [T, W]");
+  const void* ep = nullptr;
+  long est = 0;
+  if (extra.has_value()) {
+    CHECK_ROWS(*extra);
+    TORCH_CHECK(act_is_f32(*extra, "extra") == f32 &&
+                    extra->size(0) == tokens && extra->size(1) == width,
+                "extra [T, W] in y's dtype");
+    ep = extra->data_ptr();
+    est = extra->stride(0);
+  }
+  check_hip(ks_combine_rows(out.data_ptr(), y.data_ptr(), index.data_ptr(),
+                            (int)top, ep, est, tokens, width, f32,
+                            current_stream()),
+            "combine_rows");
 }
 
 void clamped_swiglu(at::Tensor& out, at::Tensor& input, double alpha,
@@ -332,5 +582,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("ctx_attention_f32", &ctx_attention_f32,
         "paged causal attention, fp32 scores/weights, optional output gate");
   m.def("clamped_swiglu", &clamped_swiglu, "clamped GLU activation");
+  m.def("qk_headnorm_rope_cache", &qk_headnorm_rope_cache,
+        "per-head q/k RMS norm + rotary, optional value norm/rotation, KV scatter");
+  m.def("post_norm_add_rms_norm", &post_norm_add_rms_norm,
+        "fp32 residual += layer_scale * post-norm(delta) (+ rows, + row), then RMS norm");
+  m.def("router_topk", &router_topk, "sigmoid/softmax scores and top-k experts");
+  m.def("route_tokens", &route_tokens,
+        "fp32 router logits + sigmoid/softmax scores + top-k experts, fused");
+  m.def("gather_scale_rows", &gather_scale_rows, "out[r] = x[rows[r]] * scales[r]");
+  m.def("combine_rows", &combine_rows, "fp32 sum of indexed rows per token");
   def_sampling(m);
 }

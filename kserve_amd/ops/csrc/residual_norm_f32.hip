@@ -6,6 +6,11 @@
 //    out = residual / sqrt(mean(residual^2) + eps) * (w_offset + w).
 //    The deltas are sublayer outputs in the activation dtype; either may be
 //    absent. One kernel covers "add the previous sublayer, norm for the next".
+//  * post_norm_add_rms_norm: closes a sandwich-normed sublayer and opens the
+//    next one: residual += layer_scale * (delta / rms(delta) * post_gain),
+//    += an optional per-token row and an optional shared row, then
+//    out = residual / rms(residual) * next_gain. Both norms have ONE gain for
+//    all channels (host scalars).
 //  * gated_group_rms_norm: v = y * silu(z), normalised separately in equal
 //    contiguous groups of the row, times a weight (gate before the norm).
 //
@@ -29,8 +34,11 @@ __global__ void embed_scale_sinpos_kernel(float* __restrict__ out,
   const long tok = tokens[t];
   const float pos = (float)positions[t];
   for (int i = threadIdx.x; i < width; i += NT) {
-    const float ang = pos * inv_freq[i >> 1];
-    const float pe = (i & 1) ? cosf(ang) : sinf(ang);
+    float pe = 0.f;  // no table of frequencies: no positional term
+    if (inv_freq) {
+      const float ang = pos * inv_freq[i >> 1];
+      pe = (i & 1) ? cosf(ang) : sinf(ang);
+    }
     out[t * width + i] = ld_f32(table, tok * width + i) * scale + pe;
   }
 }
@@ -140,6 +148,113 @@ __global__ void add_rms_norm_f32res_vec4_kernel(
       ld4<float>(weight + i, w);
 #pragma unroll
       for (int j = 0; j < 4; ++j) o[j] = keep[k][j] * inv * (w_offset + w[j]);
+      st4<TO>(out + row * width + i, o);
+    }
+  }
+}
+
+template <typename TD, typename TO>
+__global__ void post_norm_add_rms_norm_kernel(
+    float* __restrict__ residual, const TD* __restrict__ delta,
+    long delta_stride, float post_gain, const float* __restrict__ layer_scale,
+    const float* __restrict__ add_rows, const float* __restrict__ add_vec,
+    float eps, float next_gain, TO* __restrict__ out, int width) {
+  __shared__ float scratch[NW];
+  const long row = blockIdx.x;
+  float* r = residual + row * width;
+  float dinv = 0.f;
+  if (delta) {
+    float sd = 0.f;
+    for (int i = threadIdx.x; i < width; i += NT) {
+      const float d = ld_f32(delta, row * delta_stride + i);
+      sd += d * d;
+    }
+    sd = block_sum_sync<NW>(sd, scratch);
+    dinv = 1.0f / sqrtf(sd / (float)width + eps);
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += NT) {
+    float v = r[i];
+    if (delta)
+      v += ld_f32(delta, row * delta_stride + i) * dinv * post_gain * layer_scale[i];
+    if (add_rows) v += add_rows[row * width + i];
+    if (add_vec) v += add_vec[i];
+    if (delta || add_rows || add_vec) r[i] = v;
+    ss += v * v;
+  }
+  if (!out) return;
+  ss = block_sum_sync<NW>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += NT)
+    // each thread re-reads only what it wrote itself
+    st_f32(out, row * width + i, r[i] * inv * next_gain);
+}
+
+template <typename TD, typename TO>
+__global__ void post_norm_add_rms_norm_vec4_kernel(
+    float* __restrict__ residual, const TD* __restrict__ delta,
+    long delta_stride, float post_gain, const float* __restrict__ layer_scale,
+    const float* __restrict__ add_rows, const float* __restrict__ add_vec,
+    float eps, float next_gain, TO* __restrict__ out, int width) {
+  __shared__ float scratch[NW];
+  const long row = blockIdx.x;
+  float* r = residual + row * width;
+  float keep[VEC_STEPS][4];
+  float dinv = 0.f;
+  if (delta) {
+    float sd = 0.f;
+#pragma unroll
+    for (int k = 0; k < VEC_STEPS; ++k) {
+      const int i = (threadIdx.x + NT * k) * 4;
+      if (i < width) {
+        ld4<TD>(delta + row * delta_stride + i, keep[k]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sd += keep[k][j] * keep[k][j];
+      }
+    }
+    sd = block_sum_sync<NW>(sd, scratch);
+    dinv = 1.0f / sqrtf(sd / (float)width + eps);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < VEC_STEPS; ++k) {
+    const int i = (threadIdx.x + NT * k) * 4;
+    if (i < width) {
+      float v[4], a[4];
+      ld4<float>(r + i, v);
+      if (delta) {
+        ld4<float>(layer_scale + i, a);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] += keep[k][j] * dinv * post_gain * a[j];
+      }
+      if (add_rows) {
+        ld4<float>(add_rows + row * width + i, a);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] += a[j];
+      }
+      if (add_vec) {
+        ld4<float>(add_vec + i, a);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] += a[j];
+      }
+      if (delta || add_rows || add_vec) st4<float>(r + i, v);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        keep[k][j] = v[j];
+        ss += v[j] * v[j];
+      }
+    }
+  }
+  if (!out) return;
+  ss = block_sum_sync<NW>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+  for (int k = 0; k < VEC_STEPS; ++k) {
+    const int i = (threadIdx.x + NT * k) * 4;
+    if (i < width) {
+      float o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = keep[k][j] * inv * next_gain;
       st4<TO>(out + row * width + i, o);
     }
   }
@@ -262,6 +377,46 @@ extern "C" hipError_t ks_add_rms_norm_f32res(
     else
       hipLaunchKernelGGL((add_rms_norm_f32res_kernel<short, short>), dim3(rows),
                          dim3(NT), 0, stream, NORM_ARGS(short));
+  }
+  HIP_CHECK_KERNEL();
+  return hipSuccess;
+}
+
+template <typename TD, typename TO>
+static void launch_post_norm(bool vec, void* residual, const void* delta,
+                             long delta_stride, float post_gain,
+                             const void* layer_scale, const void* add_rows,
+                             const void* add_vec, float eps, float next_gain,
+                             void* out, int rows, int width,
+                             hipStream_t stream) {
+  auto fn = vec ? post_norm_add_rms_norm_vec4_kernel<TD, TO>
+                : post_norm_add_rms_norm_kernel<TD, TO>;
+  hipLaunchKernelGGL(fn, dim3(rows), dim3(NT), 0, stream, (float*)residual,
+                     (const TD*)delta, delta_stride, post_gain,
+                     (const float*)layer_scale, (const float*)add_rows,
+                     (const float*)add_vec, eps, next_gain, (TO*)out, width);
+}
+
+extern "C" hipError_t ks_post_norm_add_rms_norm(
+    void* residual, const void* delta, long delta_stride, int delta_is_f32,
+    float post_gain, const void* layer_scale, const void* add_rows,
+    const void* add_vec, float eps, float next_gain, void* out, int out_is_f32,
+    int rows, int width, hipStream_t stream) {
+  if (rows == 0) return hipSuccess;
+  if (delta && !layer_scale) return hipErrorInvalidValue;
+  auto al = [](const void* p, int bytes) { return ((uintptr_t)p % bytes) == 0; };
+  const bool vec = width % 4 == 0 && width <= NT * 4 * VEC_STEPS &&
+                   delta_stride % 4 == 0 && al(residual, 16) &&
+                   al(layer_scale, 16) && al(add_rows, 16) && al(add_vec, 16) &&
+                   al(delta, delta_is_f32 ? 16 : 8) &&
+                   al(out, out_is_f32 ? 16 : 8);
+#define PN_ARGS                                                                vec, residual, delta, delta_stride, post_gain, layer_scale, add_rows,            add_vec, eps, next_gain, out, rows, width, stream
+  if (delta_is_f32) {
+    if (out_is_f32) launch_post_norm<float, float>(PN_ARGS);
+    else launch_post_norm<float, short>(PN_ARGS);
+  } else {
+    if (out_is_f32) launch_post_norm<short, float>(PN_ARGS);
+    else launch_post_norm<short, short>(PN_ARGS);
   }
   HIP_CHECK_KERNEL();
   return hipSuccess;
