@@ -203,16 +203,19 @@ class LLMEngine:
         ):
             # MoE decode captures via the dense-bmm path (static shapes);
             # buckets are capped at the dense/sparse crossover, larger
-            # batches run eager sparse steps
-            if config.model.num_local_experts > 0:
+            # batches run eager sparse steps. A model may name its own cap.
+            cap = getattr(self.model, "decode_graph_max_tokens", None)
+            if cap is None and config.model.num_local_experts > 0:
                 from kserve_amd.models.llama import MixtralMoE
 
+                cap = MixtralMoE.DENSE_MAX_TOKENS
+            if cap is not None:
                 self.runner.capture_decode_graphs(
                     batch_sizes=[
                         b
                         for b in (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128,
                                   192, 256, 384)
-                        if b <= MixtralMoE.DENSE_MAX_TOKENS
+                        if b <= cap
                     ]
                 )
             else:
