@@ -75,6 +75,57 @@ def _hybrid_model_configs(size: dict, layers: int):
     return hybrid, llama
 
 
+# layer shapes for --desalix-compare: the widths and heads of HYBRID_SIZES;
+# 8 experts of which a token uses 2, each half as wide as the dense
+# feed-forward of that size, so a token does the arithmetic of the dense
+# layer; attention is local to `chunk` positions
+DESALIX_SIZES = {
+    "2k": dict(width=2048, heads=16, kv_heads=4, head_dim=128, ff=4096,
+               experts=8, top=2, chunk=1024, vocab=32000),
+    "4k": dict(width=4096, heads=32, kv_heads=8, head_dim=128, ff=7168,
+               experts=8, top=2, chunk=1024, vocab=32000),
+}
+
+
+def _desalix_model_configs(size: dict, runs: int):
+    """A Desalix model whose middle layer is run ``runs - 2`` times (so a
+    token passes ``runs`` layers) and a llama model of ``runs`` layers with
+    the same width and heads and a dense feed-forward as wide as the experts
+    one token uses (equal arithmetic per token; full causal attention, whose
+    work per query grows with the context while the chunk-local one's does
+    not)."""
+    from kserve_amd.engine.config import (
+        AttentionMixerSpec,
+        HybridLayerSpec,
+        HybridModelConfig,
+        LoopSpec,
+        ModelConfig,
+        MoESpec,
+    )
+
+    attn = AttentionMixerSpec(heads=size["heads"], kv_heads=size["kv_heads"],
+                              dim=size["head_dim"], vdim=size["head_dim"],
+                              scale=size["head_dim"] ** -0.5,
+                              rot_dims=size["head_dim"] // 2, rot_base=500000.0,
+                              chunk=size["chunk"])
+    mlp = MoESpec(experts=size["experts"], top=size["top"], ff=size["ff"],
+                  limit=7.0, shared=None)
+    desalix = HybridModelConfig(
+        vocab_size=size["vocab"], hidden_size=size["width"],
+        layers=[HybridLayerSpec("attention", attention=attn, mlp=mlp)
+                for _ in range(3)],
+        loop=LoopSpec(start=1, stop=2, times=runs - 2),
+        model_name="desalix-bench", architecture="Desalix",
+    )
+    llama = ModelConfig(vocab_size=size["vocab"], hidden_size=size["width"],
+                        intermediate_size=size["top"] * size["ff"],
+                        num_layers=runs,
+                        num_heads=size["heads"], num_kv_heads=size["kv_heads"],
+                        head_dim=size["head_dim"],
+                        max_position_embeddings=8192, model_name="llama-bench")
+    return desalix, llama
+
+
 def _throughput(mcfg, prompt_len, n_prompts, concurrency, steps, warmup, eager):
     """(prefill tok/s, decode tok/s) through the engine's own step()."""
     import torch
@@ -168,6 +219,58 @@ def hybrid_compare(args):
             }), flush=True)
 
 
+def desalix_compare(args):
+    """Prefill and decode tok/s of the Desalix design next to a llama model of
+    equal width, heads, depth and feed-forward arithmetic per token, both
+    through LLMEngine.step() on one GPU, bf16, random weights. One JSON line per
+    (size, model), each measured in a process of its own and printed as soon
+    as it is done."""
+    import subprocess
+    import sys
+
+    if args.compare_only is None or "," in args.desalix_compare:
+        rc = 0
+        for name in args.desalix_compare.split(","):
+            for label in ("desalix", "llama"):
+                if args.compare_only and args.compare_only != label:
+                    continue
+                cmd = [sys.executable, "-u", os.path.abspath(__file__),
+                       "--desalix-compare", name, "--compare-only", label,
+                       "--steps", str(args.steps), "--warmup", str(args.warmup),
+                       "--concurrency", str(args.concurrency),
+                       "--prompt-len", str(args.prompt_len)]
+                if args.eager:
+                    cmd.append("--eager")
+                rc = subprocess.call(cmd)
+                if rc != 0:
+                    return rc
+        return rc
+
+    import torch
+
+    assert torch.cuda.is_available(), "--desalix-compare needs a GPU"
+    name, label = args.desalix_compare, args.compare_only
+    size = DESALIX_SIZES[name]
+    desalix, llama = _desalix_model_configs(size, runs=4)
+    mcfg = desalix if label == "desalix" else llama
+    prefill, decode = _throughput(
+        mcfg, prompt_len=args.prompt_len if args.prompt_len != 512 else 2048,
+        n_prompts=8, concurrency=min(args.concurrency, 256),
+        steps=args.steps, warmup=args.warmup, eager=args.eager,
+    )
+    print(json.dumps({
+        "bench": "desalix-compare", "size": name, "model": mcfg.model_name,
+        "layer_runs": 4, "width": size["width"],
+        "experts": size["experts"], "top": size["top"],
+        "prefill_tok_s": round(prefill, 1),
+        "decode_tok_s": round(decode, 1),
+        "prefill_batch": "8 x prompt", "decode_concurrency":
+            min(args.concurrency, 256),
+        "dtype": "bfloat16", "data": "synthetic, random-init weights",
+    }), flush=True)
+    return 0
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -206,11 +309,24 @@ def main():
                         choices=["hybrid", "llama"],
                         help="with --hybrid-compare: run one side only "
                              "(e.g. under a profiler)")
+    parser.add_argument("--desalix-compare", type=str, default=None,
+                        metavar="SIZE[,SIZE...]",
+                        help="instead of the flagship workload: prefill and "
+                             "decode throughput of a Desalix-design model "
+                             "beside a llama model of equal width, heads, "
+                             "depth and arithmetic per token (sizes: "
+                             + ", ".join(DESALIX_SIZES) + ")")
+    parser.add_argument("--compare-only", type=str, default=None,
+                        choices=["desalix", "llama"],
+                        help="with --desalix-compare: run one side only "
+                             "(e.g. under a profiler)")
     parser.add_argument("--profile-cpu", action="store_true",
                         help="cProfile the timed loop and print hot functions")
     args = parser.parse_args()
     if args.hybrid_compare:
         return hybrid_compare(args)
+    if args.desalix_compare:
+        return desalix_compare(args)
 
     import torch
 
